@@ -1,0 +1,119 @@
+"""Forward of the oracle pinned against independent statements."""
+import pytest
+import torch
+
+from oracle import na2d_oracle as O
+
+
+def _rand(shape, seed=0, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(shape, generator=g, dtype=torch.float32).to(dtype) for _ in range(3)]
+
+
+@pytest.mark.parametrize("shape,k", [((1, 1, 5, 6, 4), 3), ((1, 2, 6, 5, 3), 5), ((1, 1, 7, 7, 2), 7)])
+def test_gather_matches_brute_force(shape, k):
+    q, kk, v = _rand(shape, 1)
+    o, lse = O.natten2d_gather(q, kk, v, k, return_lse=True)
+    ob, lb = O.natten2d_brute(q, kk, v, k)
+    assert O.max_abs_err(o, ob) < 1e-12
+    assert O.max_abs_err(lse, lb) < 1e-12
+
+
+@pytest.mark.parametrize("k", [3, 5, 7, 9, 11, 13])
+@pytest.mark.parametrize("hw", [(16, 16), (13, 19)])
+def test_gather_matches_dense_mask_sdpa(k, hw):
+    H, W = hw
+    if min(H, W) < k:
+        pytest.skip("image smaller than window")
+    q, kk, v = _rand((2, 2, H, W, 8), 2)
+    o = O.natten2d_gather(q, kk, v, k)
+    od = O.natten2d_dense_mask(q, kk, v, k)
+    assert O.max_abs_err(o, od) < 1e-11
+
+
+def test_scale_argument():
+    q, kk, v = _rand((1, 2, 8, 8, 16), 3)
+    a = O.natten2d_gather(q, kk, v, 3, scale=0.25)
+    b = O.natten2d_gather(q * 0.25, kk, v, 3)
+    c = O.natten2d_dense_mask(q, kk, v, 3, scale=0.25)
+    assert O.max_abs_err(a, b) < 1e-12
+    assert O.max_abs_err(a, c) < 1e-12
+
+
+def test_k1_returns_v():
+    q, kk, v = _rand((2, 1, 4, 5, 3), 4)
+    o, lse = O.natten2d_gather(q, kk, v, 1, return_lse=True)
+    assert O.max_abs_err(o, v) < 1e-14
+    assert O.max_abs_err(lse, (q * kk).sum(-1)) < 1e-12
+
+
+def test_full_window_is_global_attention():
+    q, kk, v = _rand((1, 2, 5, 5, 4), 5)
+    o = O.natten2d_gather(q, kk, v, 5)
+    f = lambda t: t.reshape(1, 2, 25, 4)
+    p = torch.softmax(f(q) @ f(kk).transpose(-1, -2), dim=-1)
+    assert O.max_abs_err(o, (p @ f(v)).reshape(1, 2, 5, 5, 4)) < 1e-12
+
+
+def test_invariances():
+    q, kk, v = _rand((1, 2, 9, 10, 6), 6)
+    o = O.natten2d_gather(q, kk, v, 5)
+    # constant V -> constant O
+    vc = torch.ones_like(v) * 3.5
+    assert O.max_abs_err(O.natten2d_gather(q, kk, vc, 5), vc) < 1e-12
+    # adding one vector to every key shifts all logits of a query equally
+    shift = torch.randn(6, dtype=torch.float64)
+    assert O.max_abs_err(O.natten2d_gather(q, kk + shift, v, 5), o) < 1e-10
+    # flips and transposition of the image axes commute with the operator
+    fl = lambda t: t.flip(2)
+    assert O.max_abs_err(O.natten2d_gather(fl(q), fl(kk), fl(v), 5), fl(o)) < 1e-12
+    tr = lambda t: t.transpose(2, 3)
+    assert O.max_abs_err(O.natten2d_gather(tr(q), tr(kk), tr(v), 5), tr(o)) < 1e-12
+
+
+@pytest.mark.parametrize("k", [3, 5, 7, 9])
+def test_loop_restatement_clean_equals_gather(k):
+    q, kk, v = _rand((2, 2, 11, 13, 4), 7)
+    o = O.natten2d_gather(q, kk, v, k)
+    ol = O.natten2d_loops(q, kk, v, k)
+    assert O.max_abs_err(o, ol) < 1e-12
+
+
+def test_loop_restatement_row_band():
+    q, kk, v = _rand((1, 1, 12, 9, 4), 8)
+    o = O.natten2d_gather(q, kk, v, 5)
+    ol = O.natten2d_loops(q, kk, v, 5, False, (4, 8))
+    assert O.max_abs_err(o[:, :, 4:8], ol[:, :, 4:8]) < 1e-12
+    assert ol[:, :, :4].abs().max() == 0 and ol[:, :, 8:].abs().max() == 0
+
+
+def test_loop_restatement_quirks_mode_differs_only_where_predicted():
+    # k=5: k//2 = 2 ... the literal offset rule is exact for k in {5, 7, 11, 13}
+    q, kk, v = _rand((1, 1, 16, 16, 4), 9)
+    o = O.natten2d_gather(q, kk, v, 5)
+    assert O.max_abs_err(O.natten2d_loops(q, kk, v, 5, True), o) < 1e-12
+    # k=3: rows/cols with index 2 pick a window shifted by one
+    o3 = O.natten2d_gather(q, kk, v, 3)
+    ol3 = O.natten2d_loops(q, kk, v, 3, True)
+    bad = (o3 - ol3).abs().amax(dim=(0, 1, 4)) > 1e-9
+    expect = torch.zeros(16, 16, dtype=torch.bool)
+    expect[2, :] = True
+    expect[:, 2] = True
+    assert torch.equal(bad, expect)
+
+
+@pytest.mark.parametrize("shape,k", [((2, 3, 16, 16, 2), 3), ((1, 2, 14, 14, 32), 7), ((1, 1, 20, 17, 8), 13)])
+def test_c_oracle_forward(shape, k, c_oracle):
+    q, kk, v = _rand(shape, 10, torch.float32)
+    o, lse = O.natten2d_gather(q.double(), kk.double(), v.double(), k, return_lse=True)
+    oc, lc = c_oracle.forward(q, kk, v, k)
+    assert O.max_abs_err(oc, o) < 2e-6
+    assert O.max_abs_err(lc, lse) < 4e-6
+
+
+def test_unfused_comparator_equals_fused():
+    # the procedure of the reference's test.py:16-21: qk -> softmax -> av
+    q, kk, v = _rand((2, 6, 16, 16, 2), 0)
+    for k in [3, 5, 7, 9, 11]:
+        p = torch.softmax(O.natten2d_qk(q, kk, k), dim=-1)
+        assert O.max_abs_err(O.natten2d_av(p, v, k), O.natten2d_gather(q, kk, v, k)) < 1e-12
