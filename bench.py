@@ -1,0 +1,181 @@
+"""Benchmark of the fused 2D neighborhood attention hot path on one MI355X.
+
+A step is one forward + backward of ``natten2d`` (through the autograd Function
+and the C ABI) on the reference's benchmark shape (bench.py:14,39 of the
+reference: B=4, heads=4, head_dim=128, kernel_size=5) in bf16 at image side 128.
+Prints ONE JSON line.  `value` is useful TFLOP/s (14*k^2*d FLOP per query);
+`roofline` is the achieved algorithmic HBM bandwidth of the slowest kernel, from
+HIP events recorded around every kernel launch inside the timed region;
+`cpu_baseline` times the CPU restatement of the reference's algorithm on this
+machine's host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TF = 2500.0   # dense bf16, published
+KERNELS = ("fwd", "bwd_dq", "bwd_dkdv")
+
+
+def algorithmic_bytes(B, N, H, W, D, esize):
+    """Bytes each kernel must move at minimum, per launch.
+    fwd : read q,k,v, write o (+ 4 B/query log-sum-exp)
+    dq  : read q,k,v,dO (+ lse), write dq
+    dkdv: read q,k,v,dO (+ lse), write dk,dv
+    path: 11*M*s + 8*q, the fused-backward minimum (q,k,v,dO read once in bwd)."""
+    q = B * N * H * W
+    M = q * D * esize
+    return {"fwd": 4 * M + 4 * q, "bwd_dq": 5 * M + 4 * q, "bwd_dkdv": 6 * M + 4 * q,
+            "path": 11 * M + 8 * q}
+
+
+def cpu_baseline(shape, ks, dtype, useful_flop, budget_rows=8):
+    """Times the CPU restatements on this host.  The headline figure is the
+    loop port of the reference's algorithm (its Python loops, softmax Jacobian
+    and inverse-neighbourhood gather) on a band of image rows, scaled to the
+    whole image; the vectorised and C/OpenMP oracles are timed on the full
+    workload beside it."""
+    import torch
+    from oracle import na2d_c, na2d_oracle as O
+    B, N, H, W, D = shape
+    g = torch.Generator().manual_seed(0)
+    q, k, v, d_o = (torch.randn(shape, generator=g).to(dtype).float() for _ in range(4))
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(min(cores, 16))
+    threads = torch.get_num_threads()
+
+    r0 = (H // 2) - (H // 2) % 3
+    r1 = min(H, r0 + budget_rows)
+    qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+    t0 = time.perf_counter()
+    o = O.natten2d_loops(qq, kk, vv, ks, False, (r0, r1))
+    o.backward(d_o)
+    loops_s = (time.perf_counter() - t0) * H / (r1 - r0)
+
+    t0 = time.perf_counter()
+    O.natten2d_gather_grads(q, k, v, d_o, ks, compute_dtype=torch.float32)
+    vec_s = time.perf_counter() - t0
+
+    na2d_c.lib()
+    t0 = time.perf_counter()
+    na2d_c.forward(q, k, v, ks, nthreads=threads)
+    na2d_c.backward(q, k, v, d_o, ks, nthreads=threads)
+    c_s = time.perf_counter() - t0
+    return {
+        "value": useful_flop / loops_s / 1e12, "unit": "TFLOP/s", "cores": threads,
+        "kind": "port", "ms": loops_s * 1e3,
+        "sample": "loop port of the reference algorithm, fp32, query/key rows %d..%d of %d "
+                  "(all %d batch*head slabs), time scaled by %d/%d" % (r0, r1 - 1, H, B * N, H, r1 - r0),
+        "vectorised_gather_ms": vec_s * 1e3, "c_openmp_ms": c_s * 1e3,
+        "host_cpus": cores,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--side", type=int, default=128)
+    ap.add_argument("--batch", type=int, default=4)
+    ap.add_argument("--heads", type=int, default=4)
+    ap.add_argument("--head-dim", type=int, default=128)
+    ap.add_argument("--kernel-size", type=int, default=5)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--simt", action="store_true", help="force the vector-ALU kernels")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this operator is measured on one GPU only (--gpus 1); "
+                 "it has no cross-GPU path, batch*head slabs are independent")
+
+    import torch
+    from e_natten_amd import Natten2d, _lib, kernel_path
+    if not os.path.exists(_lib.LIB_PATH):
+        from e_natten_amd import build
+        build.build()
+    lib = _lib.load()
+    if args.simt:
+        lib.enatten_set_path(_lib.PATH_SIMT)
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype]
+    B, N, S, D, ks = args.batch, args.heads, args.side, args.head_dim, args.kernel_size
+    shape = (B, N, S, S, D)
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    q, k, v, d_o = (torch.randn(shape, generator=g).to(dtype).to(dev) for _ in range(4))
+    q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
+
+    def step():
+        o = Natten2d.apply(q, k, v, ks)
+        return torch.autograd.grad(o, (q, k, v), d_o)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    lib.enatten_profile_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.enatten_profile_enable(0)
+
+    ms_step = elapsed * 1e3 / args.steps
+    queries = B * N * S * S
+    useful = 14.0 * ks * ks * D * queries
+    alg = algorithmic_bytes(B, N, S, S, D, q.element_size())
+
+    kern = {}
+    for i, name in enumerate(KERNELS):
+        n, tot = ctypes.c_int(), ctypes.c_double()
+        lib.enatten_profile_read(i, ctypes.byref(n), ctypes.byref(tot))
+        avg_ms = tot.value / max(n.value, 1)
+        kern[name] = {"kernel": lib.enatten_profile_kernel_name(i).decode(), "launches": n.value,
+                      "avg_us": avg_ms * 1e3, "alg_bytes": alg[name],
+                      "GBps": alg[name] / (avg_ms * 1e-3) / 1e9 if avg_ms > 0 else 0.0}
+    dom = max(KERNELS, key=lambda n: kern[n]["avg_us"])
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        rec = json.load(open(tpath)).get("%s/side%d/%s" % (kern[dom]["kernel"], S, args.dtype))
+        traffic = rec["bytes_per_launch"] if rec else None
+    kernel_ms = sum(kern[n]["avg_us"] for n in KERNELS) / 1e3
+    roofline = {
+        "bound": "hbm", "kernel": kern[dom]["kernel"], "achieved": kern[dom]["GBps"],
+        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": kern[dom]["GBps"] / HBM_PEAK_GBS,
+        "traffic": traffic, "kernels": kern,
+        "path_alg_bytes": alg["path"], "path_kernel_ms": kernel_ms,
+        "path_GBps": alg["path"] / (kernel_ms * 1e-3) / 1e9,
+        "path_frac": alg["path"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "mfma_frac_useful": useful / (kernel_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TF,
+    }
+    out = {
+        "metric": "natten2d fwd+bwd useful TFLOP/s (B4 H4 d128 k5 bf16)",
+        "value": useful / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "natten2d fwd+bwd B=%d heads=%d H=W=%d head_dim=%d kernel_size=%d"
+                               % (B, N, S, D, ks),
+                   "kernel_path": kernel_path(D, ks, dtype), "queries": queries,
+                   "useful_gflop": useful / 1e9},
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(shape, ks, dtype, useful)
+        out["cpu_baseline"]["gpu_speedup"] = out["cpu_baseline"]["ms"] / ms_step
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,232 @@
+// C ABI of libenatten.so: argument validation and dispatch.  See enatten.h.
+
+#include <stdarg.h>
+#include <stdio.h>
+
+#include <atomic>
+#include <vector>
+
+#include "na2d_common.h"
+
+namespace enatten {
+
+static thread_local char g_err[512] = "";
+static std::atomic<int> g_path{0};
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+// ---- optional per-kernel event timing -------------------------------------
+namespace {
+struct ProfRec { hipEvent_t e0, e1; };
+struct ProfSlot {
+    std::vector<ProfRec> recs;  // events are created once and reused
+    int used = 0;
+    const char *name = "";
+};
+ProfSlot g_prof[ENATTEN_KERNEL_COUNT];
+bool g_prof_on = false;
+constexpr int kProfMax = 8192;
+}  // namespace
+
+ProfScope::ProfScope(int kernel_slot, const char *kernel_name, hipStream_t stream)
+    : slot(kernel_slot), st(stream), rec(nullptr) {
+    g_prof[slot].name = kernel_name;
+    if (!g_prof_on) return;
+    ProfSlot &ps = g_prof[slot];
+    if (ps.used >= kProfMax) return;
+    if (ps.used == (int)ps.recs.size()) {
+        ProfRec r;
+        if (hipEventCreate(&r.e0) != hipSuccess || hipEventCreate(&r.e1) != hipSuccess) return;
+        ps.recs.push_back(r);
+    }
+    ProfRec *r = &ps.recs[ps.used];
+    if (hipEventRecord(r->e0, st) != hipSuccess) return;
+    rec = r;
+}
+
+ProfScope::~ProfScope() {
+    if (!rec) return;
+    ProfRec *r = static_cast<ProfRec *>(rec);
+    if (hipEventRecord(r->e1, st) == hipSuccess) g_prof[slot].used++;
+}
+
+namespace {
+
+int elem_size(int dtype) {
+    switch (dtype) {
+        case ENATTEN_F32: return 4;
+        case ENATTEN_BF16:
+        case ENATTEN_F16: return 2;
+    }
+    return 0;
+}
+
+int check_shape(const char *fn, int B, int N, int H, int W, int D, int ks, int dtype) {
+    if (elem_size(dtype) == 0) {
+        set_error("%s: unknown dtype code %d (expected ENATTEN_F32/BF16/F16)", fn, dtype);
+        return ENATTEN_EINVAL;
+    }
+    if (B < 1 || N < 1 || H < 1 || W < 1 || D < 1) {
+        set_error("%s: every dimension must be >= 1, got B=%d heads=%d H=%d W=%d D=%d", fn, B, N,
+                  H, W, D);
+        return ENATTEN_EINVAL;
+    }
+    if (ks < 1 || ks % 2 == 0) {
+        set_error("%s: kernel_size must be odd and >= 1, got %d", fn, ks);
+        return ENATTEN_EINVAL;
+    }
+    if (H < ks || W < ks) {
+        set_error("%s: image %dx%d is smaller than kernel_size %d", fn, H, W, ks);
+        return ENATTEN_EINVAL;
+    }
+    if ((int64_t)B * N * H * W * D >= ((int64_t)1 << 40)) {
+        set_error("%s: tensor too large", fn);
+        return ENATTEN_EUNSUPPORTED;
+    }
+    return ENATTEN_OK;
+}
+
+int make_view(const char *fn, const char *name, const void *p, const int64_t *st, int N, int H,
+              int W, int D, View *out) {
+    if (!p) {
+        set_error("%s: %s is NULL", fn, name);
+        return ENATTEN_EINVAL;
+    }
+    out->ptr = p;
+    if (st) {
+        out->sb = st[0]; out->sn = st[1]; out->sh = st[2]; out->sw = st[3];
+        if (out->sb < 0 || out->sn < 0 || out->sh < 0 || out->sw < 0) {
+            set_error("%s: negative stride for %s", fn, name);
+            return ENATTEN_EINVAL;
+        }
+    } else {
+        out->sw = D;
+        out->sh = (int64_t)W * D;
+        out->sn = (int64_t)H * W * D;
+        out->sb = (int64_t)N * H * W * D;
+    }
+    return ENATTEN_OK;
+}
+
+bool use_mfma(int D, int ks, int dtype) {
+    return g_path.load() != ENATTEN_PATH_SIMT && mfma_supported(D, ks, dtype);
+}
+
+}  // namespace
+}  // namespace enatten
+
+using namespace enatten;
+
+extern "C" {
+#pragma GCC visibility push(default)
+
+int enatten_abi_version(void) { return ENATTEN_ABI_VERSION; }
+
+const char *enatten_last_error(void) { return g_err; }
+
+int enatten2d_kernel_path(int D, int kernel_size, int dtype) {
+    if (elem_size(dtype) == 0 || D < 1 || D > 1024 || kernel_size < 1 || kernel_size % 2 == 0)
+        return ENATTEN_PATH_NONE;
+    return use_mfma(D, kernel_size, dtype) ? ENATTEN_PATH_MFMA : ENATTEN_PATH_SIMT;
+}
+
+int enatten_set_path(int path) {
+    if (path != 0 && path != ENATTEN_PATH_SIMT) return g_path.load();
+    return g_path.exchange(path);
+}
+
+int enatten2d_fwd(const void *q, const void *k, const void *v, void *o, float *lse, int B,
+                  int heads, int H, int W, int D, int kernel_size, int dtype,
+                  const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                  float scale, void *stream) {
+    const char *fn = "enatten2d_fwd";
+    int rc = check_shape(fn, B, heads, H, W, D, kernel_size, dtype);
+    if (rc) return rc;
+    FwdArgs a;
+    if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
+    if ((rc = make_view(fn, "k", k, k_strides, heads, H, W, D, &a.k))) return rc;
+    if ((rc = make_view(fn, "v", v, v_strides, heads, H, W, D, &a.v))) return rc;
+    if (!o) {
+        set_error("%s: o is NULL", fn);
+        return ENATTEN_EINVAL;
+    }
+    a.o = o;
+    a.lse = lse;
+    a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (use_mfma(D, kernel_size, dtype)) return launch_fwd_mfma(a, dtype, st);
+    return launch_fwd_simt(a, dtype, st);
+}
+
+size_t enatten2d_bwd_workspace_bytes(int B, int heads, int H, int W) {
+    if (B < 1 || heads < 1 || H < 1 || W < 1) return 0;
+    return (size_t)B * heads * H * W * 2 * sizeof(float);
+}
+
+int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                  const float *lse, void *dq, void *dk, void *dv, void *workspace, int B,
+                  int heads, int H, int W, int D, int kernel_size, int dtype,
+                  const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                  float scale, void *stream) {
+    const char *fn = "enatten2d_bwd";
+    int rc = check_shape(fn, B, heads, H, W, D, kernel_size, dtype);
+    if (rc) return rc;
+    BwdArgs a;
+    if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
+    if ((rc = make_view(fn, "k", k, k_strides, heads, H, W, D, &a.k))) return rc;
+    if ((rc = make_view(fn, "v", v, v_strides, heads, H, W, D, &a.v))) return rc;
+    if (!o || !d_o || !lse || !dq || !dk || !dv || !workspace) {
+        set_error("%s: o, d_o, lse, dq, dk, dv and workspace must all be non-NULL", fn);
+        return ENATTEN_EINVAL;
+    }
+    a.o = o; a.d_o = d_o; a.lse = lse;
+    a.dq = dq; a.dk = dk; a.dv = dv;
+    a.delta = static_cast<float *>(workspace);
+    a.zinv = a.delta + (size_t)B * heads * H * W;
+    a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (use_mfma(D, kernel_size, dtype)) return launch_bwd_mfma(a, dtype, st);
+    return launch_bwd_simt(a, dtype, st);
+}
+
+int enatten_profile_enable(int on) {
+    const int prev = g_prof_on ? 1 : 0;
+    if (on)
+        for (auto &ps : g_prof) ps.used = 0;
+    g_prof_on = on != 0;
+    return prev;
+}
+
+int enatten_profile_read(int kernel, int *launches, double *total_ms) {
+    if (kernel < 0 || kernel >= ENATTEN_KERNEL_COUNT || !launches || !total_ms) {
+        set_error("enatten_profile_read: bad arguments");
+        return ENATTEN_EINVAL;
+    }
+    ProfSlot &ps = g_prof[kernel];
+    double sum = 0.0;
+    for (int i = 0; i < ps.used; i++) {
+        float ms = 0.f;
+        if (hipEventSynchronize(ps.recs[i].e1) != hipSuccess ||
+            hipEventElapsedTime(&ms, ps.recs[i].e0, ps.recs[i].e1) != hipSuccess) {
+            set_error("enatten_profile_read: event query failed");
+            return ENATTEN_ELAUNCH;
+        }
+        sum += ms;
+    }
+    *launches = ps.used;
+    *total_ms = sum;
+    return ENATTEN_OK;
+}
+
+const char *enatten_profile_kernel_name(int kernel) {
+    if (kernel < 0 || kernel >= ENATTEN_KERNEL_COUNT) return "";
+    return g_prof[kernel].name;
+}
+
+#pragma GCC visibility pop
+}  // extern "C"

@@ -1,0 +1,74 @@
+// Shared declarations of the neighborhood-attention kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "enatten.h"
+
+namespace enatten {
+
+// A [B, heads, H, W, D] tensor with unit stride on D; strides in elements.
+struct View {
+    const void *ptr;
+    int64_t sb, sn, sh, sw;
+};
+
+struct Shape {
+    int B, N, H, W, D;
+    int kh, kw;  // window extent on rows / columns (kh == kw for the 2D operator)
+    float scale;
+};
+
+struct FwdArgs {
+    View q, k, v;
+    void *o;     // contiguous
+    float *lse;  // contiguous [B, N, H, W] or nullptr
+    Shape s;
+};
+
+struct BwdArgs {
+    View q, k, v;
+    const void *o, *d_o;  // contiguous
+    const float *lse;
+    void *dq, *dk, *dv;  // contiguous
+    float *delta;        // scratch [B, N, H, W]: sum_j P_j dP_j per query
+    float *zinv;         // scratch [B, N, H, W]: 1 / sum_j exp(S_j - lse) (vector-ALU kernels)
+    Shape s;
+};
+
+// NATTEN window start on an axis of length L: centred, shifted to stay inside
+// (e_natten/pytorch.py:7-11, e_natten/triton.py:7-12).
+__host__ __device__ inline int win_start(int i, int L, int k) {
+    int s = i - (k >> 1);
+    s = s < 0 ? 0 : s;
+    return s > L - k ? L - k : s;
+}
+// Queries whose window contains key i form [inv_lo, inv_hi)
+// (e_natten/pytorch.py:13-23).
+__host__ __device__ inline int inv_lo(int i, int k) { return i < k ? 0 : i - (k >> 1); }
+__host__ __device__ inline int inv_hi(int i, int L, int k) {
+    return i >= L - k ? L : i + (k >> 1) + 1;
+}
+
+void set_error(const char *fmt, ...);
+
+// Brackets one kernel launch with HIP events when profiling is enabled.
+struct ProfScope {
+    int slot;
+    hipStream_t st;
+    void *rec;
+    ProfScope(int kernel_slot, const char *kernel_name, hipStream_t stream);
+    ~ProfScope();
+};
+
+// general fp32-FMA kernels: any D <= 1024, any odd window, f32 / bf16 / f16
+int launch_fwd_simt(const FwdArgs &a, int dtype, hipStream_t st);
+int launch_bwd_simt(const BwdArgs &a, int dtype, hipStream_t st);
+
+// matrix-core kernels: bf16 / f16, D in {32, 64, 128}, square odd window
+bool mfma_supported(int D, int ks, int dtype);
+int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st);
+int launch_bwd_mfma(const BwdArgs &a, int dtype, hipStream_t st);
+
+}  // namespace enatten

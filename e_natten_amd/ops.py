@@ -1,0 +1,154 @@
+"""Host side of the fused 2D neighborhood attention operator.
+
+Mirrors the reference's Python surface (e_natten/triton.py:487-550): a
+``torch.autograd.Function`` named ``Natten2d`` whose ``apply`` is exported as
+``natten2d(q, k, v, kernel_size) -> out`` for ``[B, heads, H, W, d]`` tensors.
+The device work is done by hand-written HIP kernels for gfx950 reached through
+the C ABI of libenatten.so; the two entry points are also registered as torch
+custom ops ``enatten::na2d_fwd`` / ``enatten::na2d_bwd``.  There is no CPU or
+eager fallback: tensors must live on the GPU and the library must be built.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
+
+
+def _validate(q, k, v, kernel_size: int) -> None:
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if not isinstance(t, torch.Tensor):
+            raise TypeError("%s must be a tensor" % name)
+    if q.dim() != 5:
+        raise ValueError("expected [B, heads, H, W, head_dim] tensors, got %d-D q" % q.dim())
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("q, k and v must have the same shape, got %s, %s, %s"
+                         % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError("q, k and v must share a dtype")
+    if q.dtype not in _DTYPES:
+        raise ValueError("dtype %s is not supported (float32, bfloat16, float16)" % q.dtype)
+    if k.device != q.device or v.device != q.device:
+        raise ValueError("q, k and v must be on the same device")
+    if not isinstance(kernel_size, int) or isinstance(kernel_size, bool):
+        raise TypeError("kernel_size must be an int")
+    if kernel_size < 1 or kernel_size % 2 == 0:
+        raise ValueError("kernel_size must be odd and >= 1, got %d" % kernel_size)
+    if q.shape[2] < kernel_size or q.shape[3] < kernel_size:
+        raise ValueError("image %dx%d is smaller than kernel_size %d"
+                         % (q.shape[2], q.shape[3], kernel_size))
+    if q.numel() == 0:
+        raise ValueError("empty tensors are not supported")
+    if q.shape[4] > 1024:
+        raise ValueError("head_dim %d exceeds the supported maximum of 1024" % q.shape[4])
+
+
+def _kernel_layout(t: torch.Tensor) -> torch.Tensor:
+    """The kernels take any (batch, head, row, column) strides but need unit
+    stride on the channel axis and no negative strides."""
+    if t.stride(4) != 1 and t.shape[4] != 1:
+        return t.contiguous()
+    return t
+
+
+def _require_gpu(t: torch.Tensor, what: str) -> None:
+    if t.device.type != "cuda":
+        raise RuntimeError("%s: tensors must be on the GPU; this build has no CPU path" % what)
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        msg = _lib.last_error()
+        raise (ValueError if rc == 1 else RuntimeError)(msg)
+
+
+def _fwd_impl(q, k, v, kernel_size: int, scale: float):
+    _validate(q, k, v, kernel_size)
+    _require_gpu(q, "enatten::na2d_fwd")
+    lib = _lib.load()
+    q, k, v = (_kernel_layout(t) for t in (q, k, v))
+    B, N, H, W, D = q.shape
+    o = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, N, H, W), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(lib.enatten2d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                 lse.data_ptr(), B, N, H, W, D, kernel_size, _DTYPES[q.dtype],
+                                 _lib.strides4(q), _lib.strides4(k), _lib.strides4(v),
+                                 float(scale), stream))
+    return o, lse
+
+
+def _bwd_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
+    _validate(q, k, v, kernel_size)
+    _require_gpu(q, "enatten::na2d_bwd")
+    if d_o.shape != q.shape or o.shape != q.shape:
+        raise ValueError("o and d_o must have the shape of q")
+    if d_o.dtype != q.dtype or o.dtype != q.dtype:
+        raise ValueError("o and d_o must have the dtype of q")
+    lib = _lib.load()
+    q, k, v = (_kernel_layout(t) for t in (q, k, v))
+    o, d_o, lse = o.contiguous(), d_o.contiguous(), lse.contiguous()
+    B, N, H, W, D = q.shape
+    dq = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
+    dk, dv = torch.empty_like(dq), torch.empty_like(dq)
+    ws = torch.empty(lib.enatten2d_bwd_workspace_bytes(B, N, H, W), dtype=torch.uint8,
+                     device=q.device)
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(lib.enatten2d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                 d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                 dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, kernel_size,
+                                 _DTYPES[q.dtype], _lib.strides4(q), _lib.strides4(k),
+                                 _lib.strides4(v), float(scale), stream))
+    return dq, dk, dv
+
+
+# torch custom ops: thin shims over the C ABI
+_torch_lib = torch.library.Library("enatten", "DEF")
+_torch_lib.define("na2d_fwd(Tensor q, Tensor k, Tensor v, int kernel_size, float scale) "
+                  "-> (Tensor, Tensor)")
+_torch_lib.define("na2d_bwd(Tensor q, Tensor k, Tensor v, Tensor o, Tensor lse, Tensor d_o, "
+                  "int kernel_size, float scale) -> (Tensor, Tensor, Tensor)")
+_torch_lib.impl("na2d_fwd", _fwd_impl, "CompositeExplicitAutograd")
+_torch_lib.impl("na2d_bwd", _bwd_impl, "CompositeExplicitAutograd")
+
+
+class Natten2d(torch.autograd.Function):
+    """2D neighborhood attention, ``[B, heads, H, W, d]`` in and out.
+
+    Same contract as the reference Function (e_natten/triton.py:487-548):
+    ``forward(ctx, Q, K, V, kernel_size=7)``; ``backward`` returns
+    ``(dQ, dK, dV, None)``.  The logits carry no softmax scale, as in the
+    reference; the optional fifth argument ``scale`` multiplies them.  The
+    forward also keeps each query's log-sum-exp so the backward can recompute
+    the probabilities without a second softmax reduction.
+    """
+
+    @staticmethod
+    def forward(ctx, Q, K, V, kernel_size=7, scale=1.0):
+        _validate(Q, K, V, kernel_size)
+        o, lse = torch.ops.enatten.na2d_fwd(Q, K, V, kernel_size, scale)
+        ctx.save_for_backward(Q, K, V, o, lse)
+        ctx.kernel_size = kernel_size
+        ctx.scale = scale
+        return o
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_output):
+        Q, K, V, o, lse = ctx.saved_tensors
+        dQ, dK, dV = torch.ops.enatten.na2d_bwd(Q, K, V, o, lse, grad_output,
+                                                 ctx.kernel_size, ctx.scale)
+        return dQ, dK, dV, None, None
+
+
+natten2d = Natten2d.apply
+
+
+def kernel_path(head_dim: int, kernel_size: int, dtype: torch.dtype) -> str:
+    """Which kernel family serves a configuration: 'mfma', 'simt' or 'none'."""
+    code = _lib.load().enatten2d_kernel_path(head_dim, kernel_size, _DTYPES.get(dtype, -1))
+    return {_lib.PATH_MFMA: "mfma", _lib.PATH_SIMT: "simt"}.get(code, "none")

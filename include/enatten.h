@@ -1,0 +1,123 @@
+/*
+ * enatten.h - C ABI of the MI355X (gfx950) neighborhood-attention library.
+ *
+ * One shared library, libenatten.so, exports exactly the functions declared
+ * here.  Every function takes raw device pointers, sizes and a HIP stream; none
+ * allocates, frees, synchronises or throws.  A non-zero return value is an error
+ * code and enatten_last_error() describes it (per calling thread).
+ *
+ * Tensor layout: [B, heads, H, W, D] as in the reference
+ * (e_natten/triton.py:489-518).  The last axis has stride 1.  q, k and v may be
+ * strided views: their element strides for the (batch, head, row, column) axes
+ * are passed as int64_t[4]; NULL means contiguous.  All other tensors are
+ * contiguous.  The logits are q.k * scale; the reference applies no scale
+ * (e_natten/triton.py:280), so drop-in callers pass 1.0f.
+ */
+#ifndef ENATTEN_H
+#define ENATTEN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ENATTEN_ABI_VERSION 1
+
+/* element types of q, k, v, o and the gradients */
+enum { ENATTEN_F32 = 0, ENATTEN_BF16 = 1, ENATTEN_F16 = 2 };
+
+/* return codes */
+enum {
+    ENATTEN_OK = 0,
+    ENATTEN_EINVAL = 1,       /* bad shape, kernel size, stride, pointer or dtype */
+    ENATTEN_EUNSUPPORTED = 2, /* valid request outside what the kernels cover */
+    ENATTEN_ELAUNCH = 3       /* the HIP runtime refused the launch */
+};
+
+/* which kernel family a call is routed to (enatten2d_kernel_path) */
+enum { ENATTEN_PATH_NONE = 0, ENATTEN_PATH_SIMT = 1, ENATTEN_PATH_MFMA = 2 };
+
+int enatten_abi_version(void);
+
+/* Message for the last non-zero return code on this thread ("" if none). */
+const char *enatten_last_error(void);
+
+/*
+ * Kernel family that would serve (D, kernel_size, dtype): ENATTEN_PATH_MFMA for
+ * the matrix-core kernels, ENATTEN_PATH_SIMT for the general fp32-FMA kernels,
+ * ENATTEN_PATH_NONE if the call would be rejected.
+ */
+int enatten2d_kernel_path(int D, int kernel_size, int dtype);
+
+/*
+ * Restrict dispatch: 0 = automatic (default), ENATTEN_PATH_SIMT = never use the
+ * matrix-core kernels.  Process-wide; meant for tests and tuning.  Returns the
+ * previous setting.
+ */
+int enatten_set_path(int path);
+
+/*
+ * Forward of 2D neighborhood attention.
+ * Replaces the launch of _attn_fwd_2d in Natten2d.forward
+ * (e_natten/triton.py:507-513; per-query math triton.py:242-302, CPU statement
+ * e_natten/pytorch.py:178-202).
+ *
+ *   o   [B, heads, H, W, D]  dtype, contiguous, fully overwritten
+ *   lse [B, heads, H, W]     float32 natural-log sum-exp of each query's scaled
+ *                            logits, contiguous; may be NULL if no backward
+ *                            will follow
+ * kernel_size is odd, 1 <= kernel_size <= min(H, W).
+ */
+int enatten2d_fwd(const void *q, const void *k, const void *v, void *o, float *lse,
+                  int B, int heads, int H, int W, int D, int kernel_size, int dtype,
+                  const int64_t *q_strides, const int64_t *k_strides,
+                  const int64_t *v_strides, float scale, void *stream);
+
+/*
+ * Bytes of device scratch enatten2d_bwd needs (two float32 per query).
+ */
+size_t enatten2d_bwd_workspace_bytes(int B, int heads, int H, int W);
+
+/*
+ * Backward of 2D neighborhood attention.
+ * Replaces the launch of _attn_bwd_2d in Natten2d.backward
+ * (e_natten/triton.py:537-546; per-query math triton.py:350-423, CPU statement
+ * e_natten/pytorch.py:228-288).  dK and dV are produced by gathering over each
+ * key's inverse neighbourhood (pytorch.py:261-270), not by atomics, so results
+ * are deterministic and the outputs need no zero-fill.
+ *
+ *   o, d_o      [B, heads, H, W, D] dtype, contiguous (forward output, upstream grad)
+ *   lse         as written by enatten2d_fwd with the same scale
+ *   dq, dk, dv  [B, heads, H, W, D] dtype, contiguous, fully overwritten
+ *   workspace   enatten2d_bwd_workspace_bytes() bytes of device memory
+ */
+int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o,
+                  const void *d_o, const float *lse, void *dq, void *dk, void *dv,
+                  void *workspace, int B, int heads, int H, int W, int D,
+                  int kernel_size, int dtype, const int64_t *q_strides,
+                  const int64_t *k_strides, const int64_t *v_strides, float scale,
+                  void *stream);
+
+/*
+ * Per-kernel timing aid for benchmarks (no counterpart in the reference, whose
+ * bench.py:28,59 times whole calls with triton.testing.do_bench).  While
+ * enabled, every kernel this library launches is bracketed by HIP events on the
+ * launch stream.  enatten_profile_enable(1) clears the records and starts,
+ * enatten_profile_enable(0) stops.  enatten_profile_read waits for the recorded
+ * events of one kernel and returns its launch count and summed duration.
+ * At most 8192 launches per kernel are recorded between two enables; further
+ * launches run untimed.  Not thread-safe; leave it off in production.
+ */
+enum { ENATTEN_KERNEL_FWD = 0, ENATTEN_KERNEL_BWD_DQ = 1, ENATTEN_KERNEL_BWD_DKDV = 2,
+       ENATTEN_KERNEL_COUNT = 3 };
+int enatten_profile_enable(int on);
+int enatten_profile_read(int kernel, int *launches, double *total_ms);
+/* Name of the device kernel last launched for that slot ("" if none yet). */
+const char *enatten_profile_kernel_name(int kernel);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ENATTEN_H */

@@ -1,0 +1,198 @@
+"""HIP kernels against the CPU oracle, through the C ABI, on a real MI355X.
+
+Tolerances: float32 within 1e-4 max-abs, bfloat16/float16 within 2e-2 of the
+reference's largest magnitude, on O, dQ, dK and dV.
+"""
+import pytest
+import torch
+
+from _util import (BF16_REL, FP32_MAX_ABS, O, assert_close, ensure_built, make_inputs,
+                   oracle_all, run_gpu)
+
+pytestmark = pytest.mark.gpu
+
+BF = torch.bfloat16
+F32 = torch.float32
+F16 = torch.float16
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _lib():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return ensure_built()
+
+
+@pytest.fixture(params=["auto", "simt"])
+def path(request, _lib):
+    prev = _lib.enatten_set_path(1 if request.param == "simt" else 0)
+    yield request.param
+    _lib.enatten_set_path(prev)
+
+
+def _case(shape, dtype, ks, seed=0, scale=1.0, q_scale=1.0, k_scale=1.0, small=False, what=""):
+    q, k, v, g = make_inputs(shape, dtype, seed, q_scale, k_scale)
+    print("case", what, shape, dtype, "k=%d" % ks, flush=True)
+    ref = oracle_all(q, k, v, g, ks, scale, small)
+    got = run_gpu(q, k, v, g, ks, scale)
+    assert_close(got, (ref[0], ref[2], ref[3], ref[4]), dtype, what)
+    return got, ref
+
+
+def test_config1_fp32_small(path):
+    # B=1, heads=2, 16x16, d=32, k=3; softmax scale d^-0.5 folded into q
+    _case((1, 2, 16, 16, 32), F32, 3, seed=0, q_scale=32 ** -0.5, small=True, what="C1")
+
+
+@pytest.mark.parametrize("ks", [3, 5, 7, 9, 11])
+def test_reference_test_procedure(ks, path):
+    # test.py:47-53: fp32 (B=2, heads=6, 16x16, d=2), loss = sum(o^2), allclose(atol=1e-5)
+    from e_natten_amd import natten2d
+    q, k, v, _ = make_inputs((2, 6, 16, 16, 2), F32, 0)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    p = torch.softmax(O.natten2d_qk(qr, kr, ks), dim=-1)
+    o_ref = O.natten2d_av(p, vr, ks)
+    (o_ref ** 2).sum().backward()
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = natten2d(qg, kg, vg, ks)
+    (o ** 2).sum().backward()
+    for x, r in ((o, o_ref), (qg.grad, qr.grad), (kg.grad, kr.grad), (vg.grad, vr.grad)):
+        assert torch.allclose(x.detach().cpu().double(), r.detach(), atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("side", [32, 64, 128])
+def test_config2_bf16_readme_shape(side, path):
+    _case((4, 4, side, side, 128), BF, 5, what="C2 side %d" % side)
+
+
+def test_config2_bf16_side256():
+    _case((4, 4, 256, 256, 128), BF, 5, what="C2 side 256")
+
+
+@pytest.mark.parametrize("side", [64, 128])
+def test_config3_fp32_readme_shape(side):
+    _case((4, 4, side, side, 128), F32, 5, what="C3 side %d" % side)
+
+
+def test_config4_large_window(path):
+    _case((2, 8, 128, 128, 64), BF, 13, what="C4")
+
+
+@pytest.mark.parametrize("heads,side", [(2, 112), (4, 56), (8, 28), (16, 14)])
+def test_config5_backbone_stages(heads, side, path):
+    s = 32 ** -0.25
+    _case((8, heads, side, side, 32), BF, 7, q_scale=s, k_scale=s, what="C5 %dx%d" % (side, side))
+
+
+@pytest.mark.parametrize("shape,ks,dtype", [
+    ((1, 1, 5, 5, 32), 5, BF),       # window == image: plain attention
+    ((2, 3, 7, 19, 64), 7, BF),      # one axis equal to the window
+    ((1, 2, 9, 23, 128), 5, BF),     # sides not multiples of any tile
+    ((1, 2, 33, 17, 128), 3, BF),
+    ((1, 2, 30, 31, 64), 9, BF),
+    ((1, 1, 26, 27, 32), 11, BF),
+    ((1, 1, 13, 13, 64), 13, BF),
+    ((2, 2, 12, 12, 32), 1, BF),     # k = 1: O == V
+    ((1, 2, 20, 18, 64), 5, F16),
+    ((1, 2, 20, 18, 128), 7, F16),
+    ((1, 3, 11, 12, 3), 3, F32),     # odd head dims: scalar loads
+    ((1, 1, 9, 9, 5), 5, BF),
+    ((1, 1, 10, 9, 48), 3, BF),
+    ((1, 1, 8, 8, 96), 5, F32),
+    ((1, 1, 8, 9, 200), 3, BF),
+    ((1, 1, 6, 6, 640), 3, F32),
+    ((1, 1, 16, 16, 256), 5, BF),
+])
+def test_edge_shapes(shape, ks, dtype, path):
+    _case(shape, dtype, ks, seed=3, small=True, what="edge")
+
+
+def test_scale_argument(path):
+    _case((1, 2, 16, 20, 64), BF, 5, scale=0.125, small=True, what="scale")
+    _case((1, 2, 12, 12, 16), F32, 3, scale=0.25, small=True, what="scale")
+
+
+def test_strided_qkv_views(path):
+    # q, k, v as views of one fused projection output [B, H, W, 3, heads, d]
+    from e_natten_amd import Natten2d
+    B, N, H, W, D, ks = 2, 4, 20, 24, 64, 5
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(B, H, W, 3, N, D, generator=g).to(BF)
+    d_o = torch.randn(B, N, H, W, D, generator=g).to(BF)
+    q, k, v = (qkv[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+    ref = oracle_all(q, k, v, d_o, ks, 1.0, small=True)
+    fused = qkv.cuda().requires_grad_(True)
+    qg, kg, vg = (fused[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+    assert not qg.is_contiguous()
+    # a non-contiguous upstream gradient as well
+    o = Natten2d.apply(qg, kg, vg, ks)
+    (o.transpose(2, 3) * d_o.cuda().transpose(2, 3)).sum().backward()
+    grads = fused.grad.cpu()
+    got = (o.detach().cpu(),) + tuple(grads[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+    assert_close(got, (ref[0], ref[2], ref[3], ref[4]), BF, "strided")
+
+
+def test_lse_matches_oracle(_lib):
+    q, k, v, g = make_inputs((1, 2, 18, 18, 64), BF, 7)
+    ref = oracle_all(q, k, v, g, 7, small=True)
+    o, lse = torch.ops.enatten.na2d_fwd(q.cuda(), k.cuda(), v.cuda(), 7, 1.0)
+    assert O.max_abs_err(lse.cpu(), ref[1]) < 1e-3
+    q, k, v, g = make_inputs((1, 2, 10, 10, 24), F32, 7)
+    ref = oracle_all(q, k, v, g, 3, small=True)
+    o, lse = torch.ops.enatten.na2d_fwd(q.cuda(), k.cuda(), v.cuda(), 3, 1.0)
+    assert O.max_abs_err(lse.cpu(), ref[1]) < 1e-5
+
+
+def test_deterministic_bitwise(path):
+    q, k, v, g = make_inputs((2, 2, 40, 40, 128), BF, 11)
+    a = run_gpu(q, k, v, g, 5)
+    b = run_gpu(q, k, v, g, 5)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+
+
+def test_full_size_invariants():
+    # properties that need no oracle, at the benchmark's full size:
+    # rows of P sum to 1  => sum_keys dV == sum_queries dO
+    # sum_j dS_j = 0      => dK summed over keys is zero up to rounding
+    # constant V          => O equals that constant
+    q, k, v, g = make_inputs((4, 4, 128, 128, 128), BF, 1)
+    o, dq, dk, dv = run_gpu(q, k, v, g, 5)
+    tot = g.float().sum((2, 3))
+    assert ((dv.float().sum((2, 3)) - tot).abs().max() / tot.abs().max()) < 2e-2
+    assert dk.float().sum((2, 3)).abs().max() / dk.float().abs().sum((2, 3)).max() < 2e-2
+    vc = torch.full_like(v, 1.5)
+    oc = run_gpu(q, k, vc, g, 5)[0]
+    assert (oc.float() - 1.5).abs().max() < 2e-2
+
+
+def test_autograd_contract(_lib):
+    from e_natten_amd import Natten2d, natten2d
+    q, k, v, g = make_inputs((1, 2, 12, 12, 32), F32, 2)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = natten2d(qg, kg, vg, 5)
+    assert o.shape == q.shape and o.dtype == q.dtype and o.device == qg.device
+    o.backward(g.cuda())
+    assert all(t.grad is not None and t.grad.shape == q.shape for t in (qg, kg, vg))
+    # default kernel size is 7, as in the reference
+    o7 = natten2d(qg, kg, vg)
+    ref7 = O.natten2d_gather(q.double(), k.double(), v.double(), 7)
+    assert O.max_abs_err(o7.detach().cpu(), ref7) < FP32_MAX_ABS
+    # no-grad call works and keeps nothing
+    with torch.no_grad():
+        o2 = natten2d(qg, kg, vg, 5)
+    assert torch.equal(o2, o.detach())
+
+
+def test_errors_on_gpu(_lib):
+    from e_natten_amd import natten2d
+    q = torch.randn(1, 1, 8, 8, 16, device="cuda")
+    with pytest.raises(ValueError):
+        natten2d(q, q, q, 4)
+    with pytest.raises(ValueError):
+        natten2d(q, q, q, 9)
+    with pytest.raises(ValueError):
+        natten2d(q, q[:, :, :4], q, 3)
+    with pytest.raises(ValueError):
+        natten2d(q.double(), q.double(), q.double(), 3)
+    with pytest.raises(ValueError):
+        natten2d(q, q.half(), q, 3)

@@ -1,0 +1,99 @@
+"""Host side and C-ABI surface, without a GPU: the library loads, exports every
+symbol the header declares, validates arguments before touching the device, and
+the Python entry points mirror the reference's signature."""
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+from _util import ROOT, ensure_built
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return ensure_built()
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "enatten.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(enatten\w*)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from e_natten_amd import _lib
+    names = _declared_functions()
+    assert "enatten2d_fwd" in names and "enatten2d_bwd" in names
+    for n in names:
+        assert hasattr(lib, n), "libenatten.so does not export %s" % n
+    assert sorted(_lib.SIGNATURES) == names
+    assert lib.enatten_abi_version() == 1
+
+
+def test_c_abi_validates_before_launch(lib):
+    from e_natten_amd import _lib
+    f = lambda ks, H=8, W=8, D=16, dt=0, q=1: lib.enatten2d_fwd(
+        q, 1, 1, 1, None, 1, 1, H, W, D, ks, dt, None, None, None, 1.0, None)
+    assert f(4) == 1 and "odd" in _lib.last_error()
+    assert f(-1) == 1
+    assert f(9) == 1 and "smaller" in _lib.last_error()
+    assert f(3, dt=7) == 1 and "dtype" in _lib.last_error()
+    assert f(3, D=0) == 1
+    assert f(3, q=None) == 1 and "NULL" in _lib.last_error()
+    assert lib.enatten2d_bwd(1, 1, 1, 1, 1, None, 1, 1, 1, 1, 1, 1, 8, 8, 16, 3, 0,
+                             None, None, None, 1.0, None) == 1
+    assert lib.enatten2d_bwd_workspace_bytes(2, 3, 4, 5) == 2 * 3 * 4 * 5 * 8
+    assert lib.enatten2d_bwd_workspace_bytes(0, 3, 4, 5) == 0
+
+
+def test_kernel_path_query(lib):
+    from e_natten_amd import kernel_path
+    assert kernel_path(128, 5, torch.float32) == "simt"
+    assert kernel_path(2, 3, torch.float32) == "simt"
+    assert kernel_path(128, 4, torch.bfloat16) == "none"
+    assert kernel_path(4096, 3, torch.bfloat16) == "none"
+    assert kernel_path(128, 5, torch.float64) == "none"
+    prev = lib.enatten_set_path(1)
+    assert kernel_path(128, 5, torch.bfloat16) == "simt"
+    lib.enatten_set_path(prev)
+
+
+def test_python_surface_mirrors_reference():
+    import e_natten_amd
+    from e_natten_amd import Natten2d, natten2d
+    # e_natten/triton.py:489: forward(ctx, Q, K, V, kernel_size=7)
+    params = list(inspect.signature(Natten2d.forward).parameters.values())
+    assert [p.name for p in params[:5]] == ["ctx", "Q", "K", "V", "kernel_size"]
+    assert params[4].default == 7
+    assert natten2d == Natten2d.apply or callable(natten2d)
+    assert "natten2d" in e_natten_amd.__all__
+
+
+def test_python_validation_without_gpu():
+    from e_natten_amd import natten2d
+    q = torch.randn(1, 1, 8, 8, 16)
+    for bad in (4, 0, 9):
+        with pytest.raises(ValueError):
+            natten2d(q, q, q, bad)
+    with pytest.raises(ValueError):
+        natten2d(q[0], q[0], q[0], 3)
+    with pytest.raises(ValueError):
+        natten2d(q, q[:, :, :4], q, 3)
+    with pytest.raises(ValueError):
+        natten2d(q.double(), q.double(), q.double(), 3)
+    with pytest.raises(TypeError):
+        natten2d(q, q, q, 3.0)
+    # valid arguments on CPU tensors: there is no CPU path, so this must fail loudly
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        natten2d(q, q, q, 3)
+
+
+def test_product_package_does_not_import_oracle():
+    pkg = os.path.join(ROOT, "e_natten_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower() or f == "never", (f, "mentions the oracle")
