@@ -95,7 +95,8 @@ struct Geo {
     static constexpr int CPR = D / 8;             // 16-byte chunks per row
     static constexpr int DS = D / 32;             // reduction steps over channels
     static constexpr int DT = D / 16;             // 16-channel MFMA row tiles of the output
-    static constexpr size_t LDS_BYTES = (size_t)2 * ROWS * PITCH * sizeof(short);
+    static constexpr size_t LDS_BYTES =
+        (size_t)2 * ROWS * PITCH * sizeof(short) + ROWS * 2 * sizeof(float);
 };
 
 // XCD-aware block order: hardware deals consecutive workgroup ids round-robin to
@@ -243,6 +244,282 @@ __global__ __launch_bounds__(256) void fwd_mfma(FwdArgs a, int tiles_r, int tile
     if (a.lse && g == 0) a.lse[tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
 }
 
+// ------------------------------------------------------------------ dQ
+// Query-centric like the forward: recompute P from the saved log-sum-exp, form
+// dP^T = V dO^T on the same halo, dS = P * (dP - delta) with delta = dO . O, and
+// dQ^T = K^T dS^T with K read back from LDS transposed.  Also writes delta for the
+// dK/dV pass.  Per-query math: e_natten/triton.py:383-398.
+template <bool BF, int D, int KS>
+__global__ __launch_bounds__(256) void bwd_dq_mfma(BwdArgs a, int tiles_r, int tiles_c,
+                                                   int nblocks) {
+    using G = Geo<D, KS>;
+    __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
+    __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
+
+    const Shape &s = a.s;
+    int t = logical_block(nblocks);
+    if (t < 0) return;
+    const int tc = t % tiles_c; t /= tiles_c;
+    const int tr = t % tiles_r;
+    const int slab = t / tiles_r;
+    const int bb = slab / s.N, nn = slab % s.N;
+    const int r0 = tr * G::TH, c0 = tc * G::TW;
+    const int hr0 = win_start(r0, s.H, KS), hc0 = win_start(c0, s.W, KS);
+
+    const short *kimg = static_cast<const short *>(a.k.ptr) + bb * a.k.sb + nn * a.k.sn;
+    const short *vimg = static_cast<const short *>(a.v.ptr) + bb * a.v.sb + nn * a.v.sn;
+    stage_halo<D, KS>(lds_k, kimg, a.k.sh, a.k.sw, hr0, hc0, s.H, s.W);
+    stage_halo<D, KS>(lds_v, vimg, a.v.sh, a.v.sw, hr0, hc0, s.H, s.W);
+    __syncthreads();
+
+    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const int wr0 = r0 + (wave >> 1) * 4, wc0 = c0 + (wave & 1) * 4;
+    if (wr0 >= s.H || wc0 >= s.W) return;
+    const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
+    const int qr = min(wr0 + (n >> 2), s.H - 1), qc = min(wc0 + (n & 3), s.W - 1);
+    const int sr0 = win_start(wr0, s.H, KS), sc0 = win_start(wc0, s.W, KS);
+    const int orow = sr0 - hr0, ocol = sc0 - hc0;
+    const int dr = win_start(qr, s.H, KS) - sr0, dc = win_start(qc, s.W, KS) - sc0;
+
+    const int64_t tok = (((int64_t)bb * s.N + nn) * s.H + qr) * s.W + qc;
+    const short *qp = static_cast<const short *>(a.q.ptr) + bb * a.q.sb + nn * a.q.sn +
+                      qr * a.q.sh + qc * a.q.sw + g * 8;
+    const short *gp = static_cast<const short *>(a.d_o) + tok * D + g * 8;
+    const short *op = static_cast<const short *>(a.o) + tok * D + g * 8;
+    s16x8 qreg[G::DS], greg[G::DS];
+    float dpart = 0.f;
+#pragma unroll
+    for (int ds = 0; ds < G::DS; ds++) {
+        qreg[ds] = *reinterpret_cast<const s16x8 *>(qp + ds * 32);
+        greg[ds] = *reinterpret_cast<const s16x8 *>(gp + ds * 32);
+        const s16x8 orow8 = *reinterpret_cast<const s16x8 *>(op + ds * 32);
+#pragma unroll
+        for (int e = 0; e < 8; e++) dpart = fmaf(cvt32<BF>(greg[ds][e]), cvt32<BF>(orow8[e]), dpart);
+    }
+    const float delta = col_sum(dpart);
+    const float lse2 = a.lse[tok] * kLog2e;
+    const float sc2 = s.scale * kLog2e;
+
+    s16x8 dsb[G::KSTEPS];
+#pragma unroll
+    for (int mt = 0; mt < G::MT; mt++) {
+        const int kk = mt * 16 + n;
+        const int row = kk < G::NK ? (orow + kk / G::SW) * G::HC + ocol + kk % G::SW : G::ZROW;
+        const short *kp = lds_k + row * G::PITCH + g * 8;
+        const short *vp = lds_v + row * G::PITCH + g * 8;
+        f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ds = 0; ds < G::DS; ds++) {
+            cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(kp + ds * 32), qreg[ds], cs);
+            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(vp + ds * 32), greg[ds], cp);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int tk = mt * 16 + g * 4 + i;
+            const int kr = tk / G::SW, kc = tk % G::SW;
+            const bool ok = tk < G::NK && (unsigned)(kr - dr) < (unsigned)KS &&
+                            (unsigned)(kc - dc) < (unsigned)KS;
+            const float p = ok ? __builtin_amdgcn_exp2f(cs[i] * sc2 - lse2) : 0.f;
+            dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - delta));
+        }
+    }
+
+    f32x4 dq[G::DT];
+#pragma unroll
+    for (int mt = 0; mt < G::DT; mt++) dq[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < G::KSTEPS; ks++) {
+        const short *kp[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
+            const int row = tk < G::NK ? (orow + tk / G::SW) * G::HC + ocol + tk % G::SW : G::ZROW;
+            kp[h] = lds_k + row * G::PITCH + (n & 3) * (D / 4);
+        }
+#pragma unroll
+        for (int mt = 0; mt < G::DT; mt++)
+            dq[mt] = mfma16<BF>(cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)),
+                                dsb[ks], dq[mt]);
+    }
+
+    if (!live) return;
+    short *dqp = static_cast<short *>(a.dq) + tok * D + g * (D / 4);
+#pragma unroll
+    for (int j = 0; j < G::DT / 2; j++) {
+        s16x8 w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[i] = cvt16<BF>(dq[2 * j][i] * s.scale);
+            w[4 + i] = cvt16<BF>(dq[2 * j + 1][i] * s.scale);
+        }
+        *reinterpret_cast<s16x8 *>(dqp + j * 8) = w;
+    }
+    if (g == 0) a.delta[tok] = delta;
+}
+
+// ------------------------------------------------------------------ dK, dV
+// Key-centric: the workgroup owns an 8x8 tile of keys and stages Q, dO, the
+// log-sum-exp and delta of the queries that attend to them, i.e. the union of the
+// keys' inverse neighbourhoods (e_natten/pytorch.py:13-23, :261-270).  That union
+// is (8+k-1)^2 queries in the interior and larger beside an image edge (the
+// clamped windows of the k//2 border queries all reach k pixels in), so it is
+// walked in blocks of at most (8+k-1)^2 queries, restaging LDS per block.  Each
+// wave owns 4x4 keys (MFMA columns) and walks the queries of the block that can
+// attend to them, 32 at a time:
+//   S = Q K^T, dP = dO V^T           (query rows from LDS, key columns in registers)
+//   P = exp(S - lse), dS = P (dP - delta), masked to the query's own window
+//   dV^T += dO^T P, dK^T += Q^T dS    (dO, Q read back from LDS transposed)
+template <bool BF, int D, int KS>
+__global__ __launch_bounds__(256) void bwd_dkdv_mfma(BwdArgs a, int tiles_r, int tiles_c,
+                                                     int nblocks) {
+    using G = Geo<D, KS>;
+    __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
+    __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
+    __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
+
+    const Shape &s = a.s;
+    int t = logical_block(nblocks);
+    if (t < 0) return;
+    const int tc = t % tiles_c; t /= tiles_c;
+    const int tr = t % tiles_r;
+    const int slab = t / tiles_r;
+    const int bb = slab / s.N, nn = slab % s.N;
+    const int r0 = tr * G::TH, c0 = tc * G::TW;
+    // queries that attend to any key of the tile
+    const int qa = inv_lo(r0, KS), qb = inv_hi(min(r0 + G::TH, s.H) - 1, s.H, KS);
+    const int ca = inv_lo(c0, KS), cb = inv_hi(min(c0 + G::TW, s.W) - 1, s.W, KS);
+
+    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const int wr0 = r0 + (wave >> 1) * 4, wc0 = c0 + (wave & 1) * 4;
+    const bool wave_on = wr0 < s.H && wc0 < s.W;
+    const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
+    const int kr = min(wr0 + (n >> 2), s.H - 1), kc = min(wc0 + (n & 3), s.W - 1);
+    // queries that attend to any key of this wave's 4x4 block
+    const int wqa = wave_on ? inv_lo(wr0, KS) : 0;
+    const int wqb = wave_on ? inv_hi(min(wr0 + 4, s.H) - 1, s.H, KS) : 0;
+    const int wca = wave_on ? inv_lo(wc0, KS) : 0;
+    const int wcb = wave_on ? inv_hi(min(wc0 + 4, s.W) - 1, s.W, KS) : 0;
+
+    const short *qimg = static_cast<const short *>(a.q.ptr) + bb * a.q.sb + nn * a.q.sn;
+    const int64_t img_tok = ((int64_t)bb * s.N + nn) * s.H * (int64_t)s.W;
+    const short *gimg = static_cast<const short *>(a.d_o) + img_tok * D;
+
+    // B operands: this lane's key, channels ds*32 + g*8 ..
+    s16x8 kreg[G::DS], vreg[G::DS];
+    {
+        const short *kp = static_cast<const short *>(a.k.ptr) + bb * a.k.sb + nn * a.k.sn +
+                          kr * a.k.sh + kc * a.k.sw + g * 8;
+        const short *vp = static_cast<const short *>(a.v.ptr) + bb * a.v.sb + nn * a.v.sn +
+                          kr * a.v.sh + kc * a.v.sw + g * 8;
+#pragma unroll
+        for (int ds = 0; ds < G::DS; ds++) {
+            kreg[ds] = *reinterpret_cast<const s16x8 *>(kp + ds * 32);
+            vreg[ds] = *reinterpret_cast<const s16x8 *>(vp + ds * 32);
+        }
+    }
+    const float sc2 = s.scale * kLog2e;
+    f32x4 dk[G::DT], dv[G::DT];
+#pragma unroll
+    for (int mt = 0; mt < G::DT; mt++) {
+        dk[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dv[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    for (int br = qa; br < qb; br += G::HR) {
+        for (int bc = ca; bc < cb; bc += G::HC) {
+            if (br != qa || bc != ca) __syncthreads();  // previous block fully consumed
+            stage_halo<D, KS>(lds_q, qimg, a.q.sh, a.q.sw, br, bc, qb, cb);
+            stage_halo<D, KS>(lds_g, gimg, (int64_t)s.W * D, D, br, bc, qb, cb);
+            for (int id = threadIdx.x; id < G::ROWS; id += 256) {
+                const int r = br + id / G::HC, c = bc + id % G::HC;
+                float2 st = make_float2(0.f, 0.f);
+                if (id < G::ZROW && r < qb && c < cb) {
+                    const int64_t qt = img_tok + (int64_t)r * s.W + c;
+                    st = make_float2(a.lse[qt] * kLog2e, a.delta[qt]);
+                }
+                lds_stat[id] = st;
+            }
+            __syncthreads();
+
+            // this wave's queries inside the staged block
+            const int ra = max(wqa, br), rb = min(wqb, br + G::HR);
+            const int cc = max(wca, bc), cd = min(wcb, bc + G::HC);
+            const int wcols = cd - cc;
+            const int nq = (rb > ra && cd > cc) ? (rb - ra) * wcols : 0;
+            const int magic = wcols > 0 ? (65536 + wcols - 1) / wcols : 0;
+            // staged row of the wave's query number qi (row-major over its rectangle)
+            auto row_of = [&](int qi, int &r, int &c) {
+                const int dvd = (qi * magic) >> 16;
+                r = ra + dvd;
+                c = cc + qi - dvd * wcols;
+                return qi < nq ? (r - br) * G::HC + (c - bc) : (int)G::ZROW;
+            };
+            for (int q0 = 0; q0 < nq; q0 += 32) {
+                s16x8 pb, dsb;
+#pragma unroll
+                for (int m2 = 0; m2 < 2; m2++) {
+                    int rr, rc;
+                    const int row = row_of(q0 + m2 * 16 + n, rr, rc);
+                    const short *qp = lds_q + row * G::PITCH + g * 8;
+                    const short *gp = lds_g + row * G::PITCH + g * 8;
+                    f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ds = 0; ds < G::DS; ds++) {
+                        cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32), kreg[ds], cs);
+                        cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32), vreg[ds], cp);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int qi = q0 + m2 * 16 + g * 4 + i;
+                        int er, ec;
+                        const int erow = row_of(qi, er, ec);
+                        const float2 st = lds_stat[erow];
+                        const bool ok = qi < nq &&
+                                        (unsigned)(kr - win_start(er, s.H, KS)) < (unsigned)KS &&
+                                        (unsigned)(kc - win_start(ec, s.W, KS)) < (unsigned)KS;
+                        const float p = ok ? __builtin_amdgcn_exp2f(cs[i] * sc2 - st.x) : 0.f;
+                        pb[m2 * 4 + i] = cvt16<BF>(p);
+                        dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
+                    }
+                }
+                const short *qt[2], *gt[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    int rr, rc;
+                    const int row = row_of(q0 + h * 16 + g * 4 + (n >> 2), rr, rc);
+                    qt[h] = lds_q + row * G::PITCH + (n & 3) * (D / 4);
+                    gt[h] = lds_g + row * G::PITCH + (n & 3) * (D / 4);
+                }
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++) {
+                    dv[mt] = mfma16<BF>(
+                        cat(lds_read_tr(gt[0] + mt * 4), lds_read_tr(gt[1] + mt * 4)), pb, dv[mt]);
+                    dk[mt] = mfma16<BF>(
+                        cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)), dsb, dk[mt]);
+                }
+            }
+        }
+    }
+
+    if (!live) return;
+    const int64_t tok = img_tok + (int64_t)kr * s.W + kc;
+    short *dkp = static_cast<short *>(a.dk) + tok * D + g * (D / 4);
+    short *dvp = static_cast<short *>(a.dv) + tok * D + g * (D / 4);
+#pragma unroll
+    for (int j = 0; j < G::DT / 2; j++) {
+        s16x8 wk, wv;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            wk[i] = cvt16<BF>(dk[2 * j][i] * s.scale);
+            wk[4 + i] = cvt16<BF>(dk[2 * j + 1][i] * s.scale);
+            wv[i] = cvt16<BF>(dv[2 * j][i]);
+            wv[4 + i] = cvt16<BF>(dv[2 * j + 1][i]);
+        }
+        *reinterpret_cast<s16x8 *>(dkp + j * 8) = wk;
+        *reinterpret_cast<s16x8 *>(dvp + j * 8) = wv;
+    }
+}
+
 // ------------------------------------------------------------------ dispatch
 template <int D, int KS>
 constexpr bool fits() {
@@ -282,6 +559,30 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
     }
 }
 
+template <bool BF, int D, int KS>
+int bwd_launch(const BwdArgs &a, hipStream_t st) {
+    if constexpr (fits<D, KS>()) {
+        using G = Geo<D, KS>;
+        const int tiles_r = (a.s.H + G::TH - 1) / G::TH, tiles_c = (a.s.W + G::TW - 1) / G::TW;
+        const int64_t nb = (int64_t)a.s.B * a.s.N * tiles_r * tiles_c;
+        const int grid = (int)((nb + 7) / 8 * 8);
+        {
+            ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
+            hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
+                               tiles_c, (int)nb);
+        }
+        {
+            ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
+            hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
+                               tiles_c, (int)nb);
+        }
+        return check_launch("enatten2d_bwd");
+    } else {
+        set_error("no matrix-core kernel for head_dim %d, kernel_size %d", D, KS);
+        return ENATTEN_EUNSUPPORTED;
+    }
+}
+
 #define ENATTEN_BY_KS(FN, BF, D, ARGS, ST)                       \
     switch ((ARGS).s.kh) {                                       \
         case 3: return FN<BF, D, 3>(ARGS, ST);                   \
@@ -301,7 +602,7 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
 
 bool fits_rt(int D, int ks) {
     const int rows = (8 + ks - 1) * (8 + ks - 1) + 1;
-    return (size_t)2 * rows * (D + 8) * 2 <= 160 * 1024;
+    return (size_t)2 * rows * (D + 8) * 2 + (size_t)rows * 8 <= 160 * 1024;
 }
 
 }  // namespace
@@ -327,7 +628,17 @@ int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st) {
 }
 
 int launch_bwd_mfma(const BwdArgs &a, int dtype, hipStream_t st) {
-    return launch_bwd_simt(a, dtype, st);
+    auto al = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (!layout_ok(a.q) || !layout_ok(a.k) || !layout_ok(a.v) || !al(a.o) || !al(a.d_o) ||
+        !al(a.dq) || !al(a.dk) || !al(a.dv))
+        return launch_bwd_simt(a, dtype, st);
+    if (dtype == ENATTEN_BF16) {
+        ENATTEN_BY_D(bwd_launch, true, a, st)
+    } else {
+        ENATTEN_BY_D(bwd_launch, false, a, st)
+    }
+    set_error("no matrix-core kernel for head_dim %d, kernel_size %d", a.s.D, a.s.kh);
+    return ENATTEN_EUNSUPPORTED;
 }
 
 }  // namespace enatten
