@@ -94,6 +94,9 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--simt", action="store_true", help="force the vector-ALU kernels")
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="also run a plain 256 MiB device copy (calibrates rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this operator is measured on one GPU only (--gpus 1); "
@@ -129,6 +132,13 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     lib.enatten_profile_enable(0)
+
+    if args.copy_calib:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     ms_step = elapsed * 1e3 / args.steps
     queries = B * N * S * S

@@ -16,6 +16,12 @@
 // g*D/4 + mt*4 + i) so that each lane ends up with D/4 contiguous channels of its
 // query and writes them with 16-byte stores.
 //
+// Scheduling: the kernels are persistent.  Each workgroup walks a strided list
+// of tiles and, while it computes one tile out of LDS, the global loads of the
+// next tile's halo are already in flight into registers; they are written to LDS
+// after the barrier that ends the current tile.  HBM latency is thus hidden
+// behind compute even when LDS only admits one or two workgroups per CU.
+//
 // Forward follows e_natten/triton.py:242-302 per query (window start, mask,
 // softmax, P.V); the log-sum-exp is kept for the backward.
 
@@ -95,153 +101,255 @@ struct Geo {
     static constexpr int CPR = D / 8;             // 16-byte chunks per row
     static constexpr int DS = D / 32;             // reduction steps over channels
     static constexpr int DT = D / 16;             // 16-channel MFMA row tiles of the output
+    static constexpr int NCH = HR * HC * CPR;     // 16-byte chunks per staged halo
+    static constexpr int NL = (NCH + 255) / 256;  // chunks per thread
+    static constexpr int NST = (ROWS + 255) / 256;  // per-query statistics per thread
     static constexpr size_t LDS_BYTES =
         (size_t)2 * ROWS * PITCH * sizeof(short) + ROWS * 2 * sizeof(float);
+    // waves per SIMD to budget registers for: one per workgroup that LDS admits
+    // on a CU (a workgroup puts one wave on each of the four SIMDs), at most 2
+    static constexpr int WAVES = 2 * LDS_BYTES <= 160 * 1024 ? 2 : 1;
 };
 
-// XCD-aware block order: hardware deals consecutive workgroup ids round-robin to
-// the 8 XCDs, each with its own L2.  Give every XCD one contiguous run of tiles
-// so the halos shared by neighbouring tiles meet in the same L2.
-__device__ inline int logical_block(int nblocks) {
-    const int per_xcd = gridDim.x >> 3;
-    const int id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    return id < nblocks ? id : -1;
+// Persistent, XCD-aware tile schedule.  Hardware deals consecutive workgroup ids
+// round-robin to the 8 XCDs, each with its own L2: every XCD gets one contiguous
+// run of tiles, and the workgroups resident on it sweep that run side by side, so
+// the halos shared by neighbouring tiles meet in the same L2.
+struct Sched {
+    int t, t_end, step;
+};
+__device__ inline Sched make_sched(int ntiles) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+    const int per = (ntiles + 7) >> 3;
+    Sched sc;
+    sc.t = xcd * per + slot;
+    sc.t_end = min(ntiles, (xcd + 1) * per);
+    sc.step = slots;
+    return sc;
 }
 
-// Copy the halo [hr0, hr0+HR) x [hc0, hc0+HC) of one image into LDS, channel-
-// major with padded pitch; positions outside the image and the spare row are
-// zero so that masked tokens contribute exact zeros to the second product.
+struct Tile {
+    int bb, nn, r0, c0;
+};
+__device__ inline Tile tile_of(int t, int tiles_r, int tiles_c, int N) {
+    Tile tl;
+    tl.c0 = (t % tiles_c) * 8; t /= tiles_c;
+    tl.r0 = (t % tiles_r) * 8; t /= tiles_r;
+    tl.bb = t / N; tl.nn = t % N;
+    return tl;
+}
+
+// Global -> registers: this thread's share of the halo [hr0, hr0+HR) x
+// [hc0, hc0+HC) of one image; positions at or beyond (rlim, clim) read as zero.
 template <int D, int KS>
-__device__ inline void stage_halo(short *lds, const short *img, int64_t sh, int64_t sw, int hr0,
-                                  int hc0, int H, int W) {
+struct HaloRegs {
+    uint4 v[Geo<D, KS>::NL];
+};
+template <int D, int KS>
+__device__ inline void halo_fetch(HaloRegs<D, KS> &reg, const short *img, int64_t sh,
+                                  int64_t sw, int hr0, int hc0, int rlim, int clim) {
     using G = Geo<D, KS>;
-    constexpr int NCH = G::HR * G::HC * G::CPR;
-    for (int id = threadIdx.x; id < NCH; id += 256) {
+#pragma unroll
+    for (int i = 0; i < G::NL; i++) {
+        const int id = threadIdx.x + i * 256;
         const int row = id / G::CPR, ch = id % G::CPR;
         const int r = hr0 + row / G::HC, c = hc0 + row % G::HC;
         uint4 v = make_uint4(0, 0, 0, 0);
-        if (r < H && c < W) v = *reinterpret_cast<const uint4 *>(img + r * sh + c * sw + ch * 8);
-        *reinterpret_cast<uint4 *>(lds + row * G::PITCH + ch * 8) = v;
+        if (id < G::NCH && r < rlim && c < clim)
+            v = *reinterpret_cast<const uint4 *>(img + r * sh + c * sw + ch * 8);
+        reg.v[i] = v;
     }
+}
+// Registers -> LDS, channel-major with padded pitch.
+template <int D, int KS>
+__device__ inline void halo_commit(short *lds, const HaloRegs<D, KS> &reg) {
+    using G = Geo<D, KS>;
+#pragma unroll
+    for (int i = 0; i < G::NL; i++) {
+        const int id = threadIdx.x + i * 256;
+        const int row = id / G::CPR, ch = id % G::CPR;
+        if (id < G::NCH) *reinterpret_cast<uint4 *>(lds + row * G::PITCH + ch * 8) = reg.v[i];
+    }
+}
+// The spare row stays zero for the whole kernel: padding tokens and tokens
+// outside a wave's halo read it, so they add exact zeros to the second product.
+template <int D, int KS>
+__device__ inline void zero_row(short *lds) {
+    using G = Geo<D, KS>;
     if (threadIdx.x < G::CPR)
         *reinterpret_cast<uint4 *>(lds + G::ZROW * G::PITCH + threadIdx.x * 8) =
             make_uint4(0, 0, 0, 0);
 }
 
+// What one lane needs to know about its query (forward, dQ) inside a tile.
+struct LaneQ {
+    bool wave_on, live;
+    int qr, qc;      // query pixel, clamped into the image
+    int orow, ocol;  // origin of the wave's halo inside the staged halo
+    int dr, dc;      // window start of this query relative to the wave's halo
+    int hr0, hc0;    // origin of the staged halo in the image
+    int64_t tok;     // flat token index of the query
+};
+template <int KS>
+__device__ inline LaneQ lane_query(const Tile &tl, const Shape &s, int wave, int n) {
+    LaneQ q;
+    const int wr0 = tl.r0 + (wave >> 1) * 4, wc0 = tl.c0 + (wave & 1) * 4;
+    q.wave_on = wr0 < s.H && wc0 < s.W;
+    q.live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
+    q.qr = min(wr0 + (n >> 2), s.H - 1);
+    q.qc = min(wc0 + (n & 3), s.W - 1);
+    q.hr0 = win_start(tl.r0, s.H, KS);
+    q.hc0 = win_start(tl.c0, s.W, KS);
+    const int sr0 = win_start(min(wr0, s.H - 1), s.H, KS);
+    const int sc0 = win_start(min(wc0, s.W - 1), s.W, KS);
+    q.orow = sr0 - q.hr0;
+    q.ocol = sc0 - q.hc0;
+    q.dr = win_start(q.qr, s.H, KS) - sr0;
+    q.dc = win_start(q.qc, s.W, KS) - sc0;
+    q.tok = (((int64_t)tl.bb * s.N + tl.nn) * s.H + q.qr) * s.W + q.qc;
+    return q;
+}
+
+template <typename T>
+__device__ inline const short *image(const View &v, const Tile &tl) {
+    return static_cast<const short *>(v.ptr) + tl.bb * v.sb + tl.nn * v.sn;
+}
+
 // ------------------------------------------------------------------ forward
 template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256) void fwd_mfma(FwdArgs a, int tiles_r, int tiles_c,
-                                                int nblocks) {
+__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
 
     const Shape &s = a.s;
-    int t = logical_block(nblocks);
-    if (t < 0) return;
-    const int tc = t % tiles_c; t /= tiles_c;
-    const int tr = t % tiles_r;
-    const int slab = t / tiles_r;
-    const int bb = slab / s.N, nn = slab % s.N;
-    const int r0 = tr * G::TH, c0 = tc * G::TW;
-    const int hr0 = win_start(r0, s.H, KS), hc0 = win_start(c0, s.W, KS);
-
-    const short *kimg = static_cast<const short *>(a.k.ptr) + bb * a.k.sb + nn * a.k.sn;
-    const short *vimg = static_cast<const short *>(a.v.ptr) + bb * a.v.sb + nn * a.v.sn;
-    stage_halo<D, KS>(lds_k, kimg, a.k.sh, a.k.sw, hr0, hc0, s.H, s.W);
-    stage_halo<D, KS>(lds_v, vimg, a.v.sh, a.v.sw, hr0, hc0, s.H, s.W);
-    __syncthreads();
+    Sched sc = make_sched(ntiles);
+    if (sc.t >= sc.t_end) return;
+    zero_row<D, KS>(lds_k);
+    zero_row<D, KS>(lds_v);
 
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
-    const int wr0 = r0 + (wave >> 1) * 4, wc0 = c0 + (wave & 1) * 4;
-    if (wr0 >= s.H || wc0 >= s.W) return;  // block of 16 queries entirely outside
-    const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
-    const int qr = min(wr0 + (n >> 2), s.H - 1), qc = min(wc0 + (n & 3), s.W - 1);
-    // origin of the wave's halo inside the image and inside the staged halo
-    const int sr0 = win_start(wr0, s.H, KS), sc0 = win_start(wc0, s.W, KS);
-    const int orow = sr0 - hr0, ocol = sc0 - hc0;
-    // this lane's query window, relative to the wave's halo
-    const int dr = win_start(qr, s.H, KS) - sr0, dc = win_start(qc, s.W, KS) - sc0;
-
-    // B operand of the first product: this lane's query, channels s*32 + g*8 ..
-    const short *qp = static_cast<const short *>(a.q.ptr) + bb * a.q.sb + nn * a.q.sn +
-                      qr * a.q.sh + qc * a.q.sw + g * 8;
-    s16x8 qreg[G::DS];
-#pragma unroll
-    for (int ds = 0; ds < G::DS; ds++) qreg[ds] = *reinterpret_cast<const s16x8 *>(qp + ds * 32);
-
-    // logits^T [halo token][query], masked, in units of log2
     const float sc2 = s.scale * kLog2e;
-    f32x4 acc[G::MT];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int mt = 0; mt < G::MT; mt++) {
-        const int kk = mt * 16 + n;
-        const int row = kk < G::NK ? (orow + kk / G::SW) * G::HC + ocol + kk % G::SW : G::ZROW;
-        const short *kp = lds_k + row * G::PITCH + g * 8;
-        f32x4 c = {0.f, 0.f, 0.f, 0.f};
+
+    // registers that carry the next tile while the current one is computed
+    HaloRegs<D, KS> kst, vst;
+    s16x8 qnext[G::DS];
+    auto prefetch = [&](const Tile &tl, const LaneQ &lq) {
+        halo_fetch<D, KS>(kst, image<short>(a.k, tl), a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W);
+        halo_fetch<D, KS>(vst, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
+        const short *qp = image<short>(a.q, tl) + lq.qr * a.q.sh + lq.qc * a.q.sw + g * 8;
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++)
-            c = mfma16<BF>(*reinterpret_cast<const s16x8 *>(kp + ds * 32), qreg[ds], c);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int tk = mt * 16 + g * 4 + i;  // halo token of accumulator row g*4+i
-            const int kr = tk / G::SW, kc = tk % G::SW;
-            const bool ok = tk < G::NK && (unsigned)(kr - dr) < (unsigned)KS &&
-                            (unsigned)(kc - dc) < (unsigned)KS;
-            c[i] = ok ? c[i] * sc2 : -INFINITY;
-            mx = fmaxf(mx, c[i]);
-        }
-        acc[mt] = c;
-    }
-    mx = col_max(mx);
-    float sum = 0.f;
-    s16x8 pb[G::KSTEPS];
-#pragma unroll
-    for (int mt = 0; mt < G::MT; mt++) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float p = __builtin_amdgcn_exp2f(acc[mt][i] - mx);
-            sum += p;
-            pb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p);
-        }
-    }
-    sum = col_sum(sum);
+            qnext[ds] = *reinterpret_cast<const s16x8 *>(qp + ds * 32);
+    };
 
-    // O^T [channel][query] = V^T P^T over the halo tokens
-    f32x4 o[G::DT];
+    Tile cur = tile_of(sc.t, tiles_r, tiles_c, s.N);
+    LaneQ lq = lane_query<KS>(cur, s, wave, n);
+    prefetch(cur, lq);
+    for (;;) {
+        halo_commit<D, KS>(lds_k, kst);
+        halo_commit<D, KS>(lds_v, vst);
+        s16x8 qreg[G::DS];
 #pragma unroll
-    for (int mt = 0; mt < G::DT; mt++) o[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < G::KSTEPS; ks++) {
-        const short *vp[2];
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
-            const int row = tk < G::NK ? (orow + tk / G::SW) * G::HC + ocol + tk % G::SW : G::ZROW;
-            vp[h] = lds_v + row * G::PITCH + (n & 3) * (D / 4);
-        }
-#pragma unroll
-        for (int mt = 0; mt < G::DT; mt++)
-            o[mt] = mfma16<BF>(cat(lds_read_tr(vp[0] + mt * 4), lds_read_tr(vp[1] + mt * 4)),
-                               pb[ks], o[mt]);
-    }
+        for (int ds = 0; ds < G::DS; ds++) qreg[ds] = qnext[ds];
+        __syncthreads();
 
-    if (!live) return;
-    const float inv = 1.f / sum;
-    const int64_t tok = (((int64_t)bb * s.N + nn) * s.H + qr) * s.W + qc;
-    short *op = static_cast<short *>(a.o) + tok * D + g * (D / 4);
-#pragma unroll
-    for (int j = 0; j < G::DT / 2; j++) {
-        s16x8 w;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            w[i] = cvt16<BF>(o[2 * j][i] * inv);
-            w[4 + i] = cvt16<BF>(o[2 * j + 1][i] * inv);
+        const int tn = sc.t + sc.step;
+        const bool more = tn < sc.t_end;
+        Tile nxt = cur;
+        LaneQ lqn = lq;
+        if (more) {
+            nxt = tile_of(tn, tiles_r, tiles_c, s.N);
+            lqn = lane_query<KS>(nxt, s, wave, n);
+            prefetch(nxt, lqn);
         }
-        *reinterpret_cast<s16x8 *>(op + j * 8) = w;
+
+        if (lq.wave_on) {
+            // logits^T [halo token][query], masked, in units of log2
+            f32x4 acc[G::MT];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int mt = 0; mt < G::MT; mt++) {
+                const int kk = mt * 16 + n;
+                const int row = kk < G::NK
+                                    ? (lq.orow + kk / G::SW) * G::HC + lq.ocol + kk % G::SW
+                                    : G::ZROW;
+                const short *kp = lds_k + row * G::PITCH + g * 8;
+                f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ds = 0; ds < G::DS; ds++)
+                    c = mfma16<BF>(*reinterpret_cast<const s16x8 *>(kp + ds * 32), qreg[ds], c);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int tk = mt * 16 + g * 4 + i;  // halo token of accumulator row g*4+i
+                    const int kr = tk / G::SW, kc = tk % G::SW;
+                    const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
+                                    (unsigned)(kc - lq.dc) < (unsigned)KS;
+                    c[i] = ok ? c[i] * sc2 : -INFINITY;
+                    mx = fmaxf(mx, c[i]);
+                }
+                acc[mt] = c;
+            }
+            mx = col_max(mx);
+            float sum = 0.f;
+            s16x8 pb[G::KSTEPS];
+#pragma unroll
+            for (int mt = 0; mt < G::MT; mt++) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float p = __builtin_amdgcn_exp2f(acc[mt][i] - mx);
+                    sum += p;
+                    pb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p);
+                }
+            }
+            sum = col_sum(sum);
+
+            // O^T [channel][query] = V^T P^T over the halo tokens
+            f32x4 o[G::DT];
+#pragma unroll
+            for (int mt = 0; mt < G::DT; mt++) o[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < G::KSTEPS; ks++) {
+                const short *vp[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
+                    const int row = tk < G::NK
+                                        ? (lq.orow + tk / G::SW) * G::HC + lq.ocol + tk % G::SW
+                                        : G::ZROW;
+                    vp[h] = lds_v + row * G::PITCH + (n & 3) * (D / 4);
+                }
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++)
+                    o[mt] = mfma16<BF>(
+                        cat(lds_read_tr(vp[0] + mt * 4), lds_read_tr(vp[1] + mt * 4)), pb[ks],
+                        o[mt]);
+            }
+
+            if (lq.live) {
+                const float inv = 1.f / sum;
+                short *op = static_cast<short *>(a.o) + lq.tok * D + g * (D / 4);
+#pragma unroll
+                for (int j = 0; j < G::DT / 2; j++) {
+                    s16x8 w;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        w[i] = cvt16<BF>(o[2 * j][i] * inv);
+                        w[4 + i] = cvt16<BF>(o[2 * j + 1][i] * inv);
+                    }
+                    *reinterpret_cast<s16x8 *>(op + j * 8) = w;
+                }
+                if (a.lse && g == 0)
+                    a.lse[lq.tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
+            }
+        }
+
+        if (!more) break;
+        __syncthreads();  // every wave is done with this tile's LDS
+        cur = nxt;
+        lq = lqn;
+        sc.t = tn;
     }
-    if (a.lse && g == 0) a.lse[tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
 }
 
 // ------------------------------------------------------------------ dQ
@@ -250,111 +358,139 @@ __global__ __launch_bounds__(256) void fwd_mfma(FwdArgs a, int tiles_r, int tile
 // dQ^T = K^T dS^T with K read back from LDS transposed.  Also writes delta for the
 // dK/dV pass.  Per-query math: e_natten/triton.py:383-398.
 template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256) void bwd_dq_mfma(BwdArgs a, int tiles_r, int tiles_c,
-                                                   int nblocks) {
+__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs a, int tiles_r, int tiles_c,
+                                                   int ntiles) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
 
     const Shape &s = a.s;
-    int t = logical_block(nblocks);
-    if (t < 0) return;
-    const int tc = t % tiles_c; t /= tiles_c;
-    const int tr = t % tiles_r;
-    const int slab = t / tiles_r;
-    const int bb = slab / s.N, nn = slab % s.N;
-    const int r0 = tr * G::TH, c0 = tc * G::TW;
-    const int hr0 = win_start(r0, s.H, KS), hc0 = win_start(c0, s.W, KS);
-
-    const short *kimg = static_cast<const short *>(a.k.ptr) + bb * a.k.sb + nn * a.k.sn;
-    const short *vimg = static_cast<const short *>(a.v.ptr) + bb * a.v.sb + nn * a.v.sn;
-    stage_halo<D, KS>(lds_k, kimg, a.k.sh, a.k.sw, hr0, hc0, s.H, s.W);
-    stage_halo<D, KS>(lds_v, vimg, a.v.sh, a.v.sw, hr0, hc0, s.H, s.W);
-    __syncthreads();
+    Sched sc = make_sched(ntiles);
+    if (sc.t >= sc.t_end) return;
+    zero_row<D, KS>(lds_k);
+    zero_row<D, KS>(lds_v);
 
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
-    const int wr0 = r0 + (wave >> 1) * 4, wc0 = c0 + (wave & 1) * 4;
-    if (wr0 >= s.H || wc0 >= s.W) return;
-    const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
-    const int qr = min(wr0 + (n >> 2), s.H - 1), qc = min(wc0 + (n & 3), s.W - 1);
-    const int sr0 = win_start(wr0, s.H, KS), sc0 = win_start(wc0, s.W, KS);
-    const int orow = sr0 - hr0, ocol = sc0 - hc0;
-    const int dr = win_start(qr, s.H, KS) - sr0, dc = win_start(qc, s.W, KS) - sc0;
-
-    const int64_t tok = (((int64_t)bb * s.N + nn) * s.H + qr) * s.W + qc;
-    const short *qp = static_cast<const short *>(a.q.ptr) + bb * a.q.sb + nn * a.q.sn +
-                      qr * a.q.sh + qc * a.q.sw + g * 8;
-    const short *gp = static_cast<const short *>(a.d_o) + tok * D + g * 8;
-    const short *op = static_cast<const short *>(a.o) + tok * D + g * 8;
-    s16x8 qreg[G::DS], greg[G::DS];
-    float dpart = 0.f;
-#pragma unroll
-    for (int ds = 0; ds < G::DS; ds++) {
-        qreg[ds] = *reinterpret_cast<const s16x8 *>(qp + ds * 32);
-        greg[ds] = *reinterpret_cast<const s16x8 *>(gp + ds * 32);
-        const s16x8 orow8 = *reinterpret_cast<const s16x8 *>(op + ds * 32);
-#pragma unroll
-        for (int e = 0; e < 8; e++) dpart = fmaf(cvt32<BF>(greg[ds][e]), cvt32<BF>(orow8[e]), dpart);
-    }
-    const float delta = col_sum(dpart);
-    const float lse2 = a.lse[tok] * kLog2e;
     const float sc2 = s.scale * kLog2e;
 
-    s16x8 dsb[G::KSTEPS];
-#pragma unroll
-    for (int mt = 0; mt < G::MT; mt++) {
-        const int kk = mt * 16 + n;
-        const int row = kk < G::NK ? (orow + kk / G::SW) * G::HC + ocol + kk % G::SW : G::ZROW;
-        const short *kp = lds_k + row * G::PITCH + g * 8;
-        const short *vp = lds_v + row * G::PITCH + g * 8;
-        f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
+    HaloRegs<D, KS> kst, vst;
+    s16x8 qnext[G::DS], gnext[G::DS], onext[G::DS];
+    float lse_next = 0.f;
+    auto prefetch = [&](const Tile &tl, const LaneQ &lq) {
+        halo_fetch<D, KS>(kst, image<short>(a.k, tl), a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W);
+        halo_fetch<D, KS>(vst, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
+        const short *qp = image<short>(a.q, tl) + lq.qr * a.q.sh + lq.qc * a.q.sw + g * 8;
+        const short *gp = static_cast<const short *>(a.d_o) + lq.tok * D + g * 8;
+        const short *op = static_cast<const short *>(a.o) + lq.tok * D + g * 8;
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) {
-            cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(kp + ds * 32), qreg[ds], cs);
-            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(vp + ds * 32), greg[ds], cp);
+            qnext[ds] = *reinterpret_cast<const s16x8 *>(qp + ds * 32);
+            gnext[ds] = *reinterpret_cast<const s16x8 *>(gp + ds * 32);
+            onext[ds] = *reinterpret_cast<const s16x8 *>(op + ds * 32);
         }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int tk = mt * 16 + g * 4 + i;
-            const int kr = tk / G::SW, kc = tk % G::SW;
-            const bool ok = tk < G::NK && (unsigned)(kr - dr) < (unsigned)KS &&
-                            (unsigned)(kc - dc) < (unsigned)KS;
-            const float p = ok ? __builtin_amdgcn_exp2f(cs[i] * sc2 - lse2) : 0.f;
-            dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - delta));
-        }
-    }
+        lse_next = a.lse[lq.tok];
+    };
 
-    f32x4 dq[G::DT];
+    Tile cur = tile_of(sc.t, tiles_r, tiles_c, s.N);
+    LaneQ lq = lane_query<KS>(cur, s, wave, n);
+    prefetch(cur, lq);
+    for (;;) {
+        halo_commit<D, KS>(lds_k, kst);
+        halo_commit<D, KS>(lds_v, vst);
+        s16x8 qreg[G::DS], greg[G::DS];
+        float dpart = 0.f;
 #pragma unroll
-    for (int mt = 0; mt < G::DT; mt++) dq[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int ds = 0; ds < G::DS; ds++) {
+            qreg[ds] = qnext[ds];
+            greg[ds] = gnext[ds];
 #pragma unroll
-    for (int ks = 0; ks < G::KSTEPS; ks++) {
-        const short *kp[2];
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
-            const int row = tk < G::NK ? (orow + tk / G::SW) * G::HC + ocol + tk % G::SW : G::ZROW;
-            kp[h] = lds_k + row * G::PITCH + (n & 3) * (D / 4);
+            for (int e = 0; e < 8; e++)
+                dpart = fmaf(cvt32<BF>(gnext[ds][e]), cvt32<BF>(onext[ds][e]), dpart);
         }
-#pragma unroll
-        for (int mt = 0; mt < G::DT; mt++)
-            dq[mt] = mfma16<BF>(cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)),
-                                dsb[ks], dq[mt]);
-    }
+        const float lse2 = lse_next * kLog2e;
+        __syncthreads();
 
-    if (!live) return;
-    short *dqp = static_cast<short *>(a.dq) + tok * D + g * (D / 4);
-#pragma unroll
-    for (int j = 0; j < G::DT / 2; j++) {
-        s16x8 w;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            w[i] = cvt16<BF>(dq[2 * j][i] * s.scale);
-            w[4 + i] = cvt16<BF>(dq[2 * j + 1][i] * s.scale);
+        const int tn = sc.t + sc.step;
+        const bool more = tn < sc.t_end;
+        Tile nxt = cur;
+        LaneQ lqn = lq;
+        if (more) {
+            nxt = tile_of(tn, tiles_r, tiles_c, s.N);
+            lqn = lane_query<KS>(nxt, s, wave, n);
+            prefetch(nxt, lqn);
         }
-        *reinterpret_cast<s16x8 *>(dqp + j * 8) = w;
+
+        if (lq.wave_on) {
+            const float delta = col_sum(dpart);
+            s16x8 dsb[G::KSTEPS];
+#pragma unroll
+            for (int mt = 0; mt < G::MT; mt++) {
+                const int kk = mt * 16 + n;
+                const int row = kk < G::NK
+                                    ? (lq.orow + kk / G::SW) * G::HC + lq.ocol + kk % G::SW
+                                    : G::ZROW;
+                const short *kp = lds_k + row * G::PITCH + g * 8;
+                const short *vp = lds_v + row * G::PITCH + g * 8;
+                f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ds = 0; ds < G::DS; ds++) {
+                    cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(kp + ds * 32), qreg[ds], cs);
+                    cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(vp + ds * 32), greg[ds], cp);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int tk = mt * 16 + g * 4 + i;
+                    const int kr = tk / G::SW, kc = tk % G::SW;
+                    const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
+                                    (unsigned)(kc - lq.dc) < (unsigned)KS;
+                    const float p = ok ? __builtin_amdgcn_exp2f(cs[i] * sc2 - lse2) : 0.f;
+                    dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - delta));
+                }
+            }
+
+            f32x4 dq[G::DT];
+#pragma unroll
+            for (int mt = 0; mt < G::DT; mt++) dq[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < G::KSTEPS; ks++) {
+                const short *kp[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
+                    const int row = tk < G::NK
+                                        ? (lq.orow + tk / G::SW) * G::HC + lq.ocol + tk % G::SW
+                                        : G::ZROW;
+                    kp[h] = lds_k + row * G::PITCH + (n & 3) * (D / 4);
+                }
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++)
+                    dq[mt] = mfma16<BF>(
+                        cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)), dsb[ks],
+                        dq[mt]);
+            }
+
+            if (lq.live) {
+                short *dqp = static_cast<short *>(a.dq) + lq.tok * D + g * (D / 4);
+#pragma unroll
+                for (int j = 0; j < G::DT / 2; j++) {
+                    s16x8 w;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        w[i] = cvt16<BF>(dq[2 * j][i] * s.scale);
+                        w[4 + i] = cvt16<BF>(dq[2 * j + 1][i] * s.scale);
+                    }
+                    *reinterpret_cast<s16x8 *>(dqp + j * 8) = w;
+                }
+                if (g == 0) a.delta[lq.tok] = delta;
+            }
+        }
+
+        if (!more) break;
+        __syncthreads();
+        cur = nxt;
+        lq = lqn;
+        sc.t = tn;
     }
-    if (g == 0) a.delta[tok] = delta;
 }
 
 // ------------------------------------------------------------------ dK, dV
@@ -363,96 +499,157 @@ __global__ __launch_bounds__(256) void bwd_dq_mfma(BwdArgs a, int tiles_r, int t
 // keys' inverse neighbourhoods (e_natten/pytorch.py:13-23, :261-270).  That union
 // is (8+k-1)^2 queries in the interior and larger beside an image edge (the
 // clamped windows of the k//2 border queries all reach k pixels in), so it is
-// walked in blocks of at most (8+k-1)^2 queries, restaging LDS per block.  Each
-// wave owns 4x4 keys (MFMA columns) and walks the queries of the block that can
-// attend to them, 32 at a time:
+// walked in blocks of at most (8+k-1)^2 queries; a block is the unit that is
+// staged in LDS and prefetched.  Each wave owns 4x4 keys (MFMA columns) and walks
+// the queries of the block that can attend to them, 32 at a time:
 //   S = Q K^T, dP = dO V^T           (query rows from LDS, key columns in registers)
 //   P = exp(S - lse), dS = P (dP - delta), masked to the query's own window
 //   dV^T += dO^T P, dK^T += Q^T dS    (dO, Q read back from LDS transposed)
+struct KeyBlock {
+    int t;                // tile
+    Tile tl;
+    int qa, qb, ca, cb;   // queries that attend to any key of the tile
+    int br, bc;           // origin of the staged block of queries
+    bool first, last;     // first / last block of its tile
+};
+template <int KS, int HR, int HC>
+__device__ inline KeyBlock first_block(int t, int tiles_r, int tiles_c, const Shape &s) {
+    KeyBlock b;
+    b.t = t;
+    b.tl = tile_of(t, tiles_r, tiles_c, s.N);
+    b.qa = inv_lo(b.tl.r0, KS);
+    b.qb = inv_hi(min(b.tl.r0 + 8, s.H) - 1, s.H, KS);
+    b.ca = inv_lo(b.tl.c0, KS);
+    b.cb = inv_hi(min(b.tl.c0 + 8, s.W) - 1, s.W, KS);
+    b.br = b.qa;
+    b.bc = b.ca;
+    b.first = true;
+    b.last = b.br + HR >= b.qb && b.bc + HC >= b.cb;
+    return b;
+}
+// Next block of the same tile, or false when the tile is finished.
+template <int HR, int HC>
+__device__ inline bool next_block(KeyBlock &b) {
+    if (b.last) return false;
+    b.first = false;
+    b.bc += HC;
+    if (b.bc >= b.cb) {
+        b.bc = b.ca;
+        b.br += HR;
+    }
+    b.last = b.br + HR >= b.qb && b.bc + HC >= b.cb;
+    return true;
+}
+
 template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256) void bwd_dkdv_mfma(BwdArgs a, int tiles_r, int tiles_c,
-                                                     int nblocks) {
+__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArgs a, int tiles_r, int tiles_c,
+                                                     int ntiles) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
     __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
 
     const Shape &s = a.s;
-    int t = logical_block(nblocks);
-    if (t < 0) return;
-    const int tc = t % tiles_c; t /= tiles_c;
-    const int tr = t % tiles_r;
-    const int slab = t / tiles_r;
-    const int bb = slab / s.N, nn = slab % s.N;
-    const int r0 = tr * G::TH, c0 = tc * G::TW;
-    // queries that attend to any key of the tile
-    const int qa = inv_lo(r0, KS), qb = inv_hi(min(r0 + G::TH, s.H) - 1, s.H, KS);
-    const int ca = inv_lo(c0, KS), cb = inv_hi(min(c0 + G::TW, s.W) - 1, s.W, KS);
+    Sched sc = make_sched(ntiles);
+    if (sc.t >= sc.t_end) return;
+    zero_row<D, KS>(lds_q);
+    zero_row<D, KS>(lds_g);
 
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
-    const int wr0 = r0 + (wave >> 1) * 4, wc0 = c0 + (wave & 1) * 4;
-    const bool wave_on = wr0 < s.H && wc0 < s.W;
-    const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
-    const int kr = min(wr0 + (n >> 2), s.H - 1), kc = min(wc0 + (n & 3), s.W - 1);
-    // queries that attend to any key of this wave's 4x4 block
-    const int wqa = wave_on ? inv_lo(wr0, KS) : 0;
-    const int wqb = wave_on ? inv_hi(min(wr0 + 4, s.H) - 1, s.H, KS) : 0;
-    const int wca = wave_on ? inv_lo(wc0, KS) : 0;
-    const int wcb = wave_on ? inv_hi(min(wc0 + 4, s.W) - 1, s.W, KS) : 0;
-
-    const short *qimg = static_cast<const short *>(a.q.ptr) + bb * a.q.sb + nn * a.q.sn;
-    const int64_t img_tok = ((int64_t)bb * s.N + nn) * s.H * (int64_t)s.W;
-    const short *gimg = static_cast<const short *>(a.d_o) + img_tok * D;
-
-    // B operands: this lane's key, channels ds*32 + g*8 ..
-    s16x8 kreg[G::DS], vreg[G::DS];
-    {
-        const short *kp = static_cast<const short *>(a.k.ptr) + bb * a.k.sb + nn * a.k.sn +
-                          kr * a.k.sh + kc * a.k.sw + g * 8;
-        const short *vp = static_cast<const short *>(a.v.ptr) + bb * a.v.sb + nn * a.v.sn +
-                          kr * a.v.sh + kc * a.v.sw + g * 8;
-#pragma unroll
-        for (int ds = 0; ds < G::DS; ds++) {
-            kreg[ds] = *reinterpret_cast<const s16x8 *>(kp + ds * 32);
-            vreg[ds] = *reinterpret_cast<const s16x8 *>(vp + ds * 32);
-        }
-    }
     const float sc2 = s.scale * kLog2e;
-    f32x4 dk[G::DT], dv[G::DT];
+
+    HaloRegs<D, KS> qst, gst;
+    float2 sst[G::NST];
+    s16x8 knext[G::DS], vnext[G::DS];
+    // the wave's 4x4 keys of a tile: this lane's key pixel (clamped into the image)
+    auto key_of = [&](const Tile &tl, int &kr, int &kc) {
+        kr = min(tl.r0 + (wave >> 1) * 4 + (n >> 2), s.H - 1);
+        kc = min(tl.c0 + (wave & 1) * 4 + (n & 3), s.W - 1);
+    };
+    auto prefetch = [&](const KeyBlock &b) {
+        const int64_t img_tok = ((int64_t)b.tl.bb * s.N + b.tl.nn) * s.H * (int64_t)s.W;
+        halo_fetch<D, KS>(qst, image<short>(a.q, b.tl), a.q.sh, a.q.sw, b.br, b.bc, b.qb, b.cb);
+        halo_fetch<D, KS>(gst, static_cast<const short *>(a.d_o) + img_tok * D, (int64_t)s.W * D,
+                          D, b.br, b.bc, b.qb, b.cb);
 #pragma unroll
-    for (int mt = 0; mt < G::DT; mt++) {
-        dk[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        dv[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-
-    for (int br = qa; br < qb; br += G::HR) {
-        for (int bc = ca; bc < cb; bc += G::HC) {
-            if (br != qa || bc != ca) __syncthreads();  // previous block fully consumed
-            stage_halo<D, KS>(lds_q, qimg, a.q.sh, a.q.sw, br, bc, qb, cb);
-            stage_halo<D, KS>(lds_g, gimg, (int64_t)s.W * D, D, br, bc, qb, cb);
-            for (int id = threadIdx.x; id < G::ROWS; id += 256) {
-                const int r = br + id / G::HC, c = bc + id % G::HC;
-                float2 st = make_float2(0.f, 0.f);
-                if (id < G::ZROW && r < qb && c < cb) {
-                    const int64_t qt = img_tok + (int64_t)r * s.W + c;
-                    st = make_float2(a.lse[qt] * kLog2e, a.delta[qt]);
-                }
-                lds_stat[id] = st;
+        for (int i = 0; i < G::NST; i++) {
+            const int id = threadIdx.x + i * 256;
+            const int r = b.br + id / G::HC, c = b.bc + id % G::HC;
+            float2 st = make_float2(0.f, 0.f);
+            if (id < G::ZROW && r < b.qb && c < b.cb) {
+                const int64_t qt = img_tok + (int64_t)r * s.W + c;
+                st = make_float2(a.lse[qt] * kLog2e, a.delta[qt]);
             }
-            __syncthreads();
+            sst[i] = st;
+        }
+        if (b.first) {
+            int kr, kc;
+            key_of(b.tl, kr, kc);
+            const short *kp = image<short>(a.k, b.tl) + kr * a.k.sh + kc * a.k.sw + g * 8;
+            const short *vp = image<short>(a.v, b.tl) + kr * a.v.sh + kc * a.v.sw + g * 8;
+#pragma unroll
+            for (int ds = 0; ds < G::DS; ds++) {
+                knext[ds] = *reinterpret_cast<const s16x8 *>(kp + ds * 32);
+                vnext[ds] = *reinterpret_cast<const s16x8 *>(vp + ds * 32);
+            }
+        }
+    };
 
-            // this wave's queries inside the staged block
-            const int ra = max(wqa, br), rb = min(wqb, br + G::HR);
-            const int cc = max(wca, bc), cd = min(wcb, bc + G::HC);
+    s16x8 kreg[G::DS], vreg[G::DS];
+    f32x4 dk[G::DT], dv[G::DT];
+    KeyBlock cur = first_block<KS, G::HR, G::HC>(sc.t, tiles_r, tiles_c, s);
+    prefetch(cur);
+    for (;;) {
+        halo_commit<D, KS>(lds_q, qst);
+        halo_commit<D, KS>(lds_g, gst);
+#pragma unroll
+        for (int i = 0; i < G::NST; i++) {
+            const int id = threadIdx.x + i * 256;
+            if (id < G::ROWS) lds_stat[id] = sst[i];
+        }
+        if (cur.first) {
+#pragma unroll
+            for (int ds = 0; ds < G::DS; ds++) {
+                kreg[ds] = knext[ds];
+                vreg[ds] = vnext[ds];
+            }
+#pragma unroll
+            for (int mt = 0; mt < G::DT; mt++) {
+                dk[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                dv[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+        __syncthreads();
+
+        KeyBlock nxt = cur;
+        bool more = next_block<G::HR, G::HC>(nxt);
+        if (!more && cur.t + sc.step < sc.t_end) {
+            nxt = first_block<KS, G::HR, G::HC>(cur.t + sc.step, tiles_r, tiles_c, s);
+            more = true;
+        }
+        if (more) prefetch(nxt);
+
+        const int wr0 = cur.tl.r0 + (wave >> 1) * 4, wc0 = cur.tl.c0 + (wave & 1) * 4;
+        const bool wave_on = wr0 < s.H && wc0 < s.W;
+        int kr, kc;
+        key_of(cur.tl, kr, kc);
+        if (wave_on) {
+            // this wave's queries inside the staged block: those that attend to any
+            // of its 4x4 keys
+            const int ra = max(inv_lo(wr0, KS), cur.br);
+            const int rb = min(inv_hi(min(wr0 + 4, s.H) - 1, s.H, KS), cur.br + G::HR);
+            const int cc = max(inv_lo(wc0, KS), cur.bc);
+            const int cd = min(inv_hi(min(wc0 + 4, s.W) - 1, s.W, KS), cur.bc + G::HC);
             const int wcols = cd - cc;
             const int nq = (rb > ra && cd > cc) ? (rb - ra) * wcols : 0;
             const int magic = wcols > 0 ? (65536 + wcols - 1) / wcols : 0;
-            // staged row of the wave's query number qi (row-major over its rectangle)
+            // staged row of the wave's query number qi (row-major over its rectangle);
+            // qi * magic >> 16 == qi / wcols for qi < 2048, wcols <= 32
             auto row_of = [&](int qi, int &r, int &c) {
                 const int dvd = (qi * magic) >> 16;
                 r = ra + dvd;
                 c = cc + qi - dvd * wcols;
-                return qi < nq ? (r - br) * G::HC + (c - bc) : (int)G::ZROW;
+                return qi < nq ? (r - cur.br) * G::HC + (c - cur.bc) : (int)G::ZROW;
             };
             for (int q0 = 0; q0 < nq; q0 += 32) {
                 s16x8 pb, dsb;
@@ -499,24 +696,31 @@ __global__ __launch_bounds__(256) void bwd_dkdv_mfma(BwdArgs a, int tiles_r, int
                 }
             }
         }
-    }
 
-    if (!live) return;
-    const int64_t tok = img_tok + (int64_t)kr * s.W + kc;
-    short *dkp = static_cast<short *>(a.dk) + tok * D + g * (D / 4);
-    short *dvp = static_cast<short *>(a.dv) + tok * D + g * (D / 4);
+        const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
+        if (cur.last && live) {
+            const int64_t tok =
+                (((int64_t)cur.tl.bb * s.N + cur.tl.nn) * s.H + kr) * s.W + kc;
+            short *dkp = static_cast<short *>(a.dk) + tok * D + g * (D / 4);
+            short *dvp = static_cast<short *>(a.dv) + tok * D + g * (D / 4);
 #pragma unroll
-    for (int j = 0; j < G::DT / 2; j++) {
-        s16x8 wk, wv;
+            for (int j = 0; j < G::DT / 2; j++) {
+                s16x8 wk, wv;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            wk[i] = cvt16<BF>(dk[2 * j][i] * s.scale);
-            wk[4 + i] = cvt16<BF>(dk[2 * j + 1][i] * s.scale);
-            wv[i] = cvt16<BF>(dv[2 * j][i]);
-            wv[4 + i] = cvt16<BF>(dv[2 * j + 1][i]);
+                for (int i = 0; i < 4; i++) {
+                    wk[i] = cvt16<BF>(dk[2 * j][i] * s.scale);
+                    wk[4 + i] = cvt16<BF>(dk[2 * j + 1][i] * s.scale);
+                    wv[i] = cvt16<BF>(dv[2 * j][i]);
+                    wv[4 + i] = cvt16<BF>(dv[2 * j + 1][i]);
+                }
+                *reinterpret_cast<s16x8 *>(dkp + j * 8) = wk;
+                *reinterpret_cast<s16x8 *>(dvp + j * 8) = wv;
+            }
         }
-        *reinterpret_cast<s16x8 *>(dkp + j * 8) = wk;
-        *reinterpret_cast<s16x8 *>(dvp + j * 8) = wv;
+
+        if (!more) break;
+        __syncthreads();
+        cur = nxt;
     }
 }
 
@@ -540,13 +744,26 @@ bool layout_ok(const View &v) {
            v.sh % 8 == 0 && v.sw % 8 == 0;
 }
 
+// Persistent grid: as many workgroups as stay resident at once (8 XCDs x 32 CUs x
+// workgroups per CU), never more than there are tiles.
+template <typename K>
+int persistent_grid(K kernel, int64_t ntiles) {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess ||
+        per_cu < 1)
+        per_cu = 1;
+    const int64_t per_xcd = (ntiles + 7) / 8;
+    const int64_t slots = per_xcd < 32 * (int64_t)per_cu ? per_xcd : 32 * (int64_t)per_cu;
+    return (int)(8 * slots);
+}
+
 template <bool BF, int D, int KS>
 int fwd_launch(const FwdArgs &a, hipStream_t st) {
     if constexpr (fits<D, KS>()) {
         using G = Geo<D, KS>;
         const int tiles_r = (a.s.H + G::TH - 1) / G::TH, tiles_c = (a.s.W + G::TW - 1) / G::TW;
         const int64_t nb = (int64_t)a.s.B * a.s.N * tiles_r * tiles_c;
-        const int grid = (int)((nb + 7) / 8 * 8);
+        const int grid = persistent_grid(fwd_mfma<BF, D, KS>, nb);
         {
             ProfScope prof(ENATTEN_KERNEL_FWD, "fwd_mfma", st);
             hipLaunchKernelGGL((fwd_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
@@ -565,13 +782,14 @@ int bwd_launch(const BwdArgs &a, hipStream_t st) {
         using G = Geo<D, KS>;
         const int tiles_r = (a.s.H + G::TH - 1) / G::TH, tiles_c = (a.s.W + G::TW - 1) / G::TW;
         const int64_t nb = (int64_t)a.s.B * a.s.N * tiles_r * tiles_c;
-        const int grid = (int)((nb + 7) / 8 * 8);
         {
+            const int grid = persistent_grid(bwd_dq_mfma<BF, D, KS>, nb);
             ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
             hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
                                tiles_c, (int)nb);
         }
         {
+            const int grid = persistent_grid(bwd_dkdv_mfma<BF, D, KS>, nb);
             ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
             hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
                                tiles_c, (int)nb);
