@@ -35,6 +35,7 @@ namespace {
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes in flight
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
@@ -42,7 +43,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
 template <bool BF>
-__device__ inline f32x4 mfma16(s16x8 a, s16x8 b, f32x4 c) {
+__device__ __forceinline__ f32x4 mfma16(s16x8 a, s16x8 b, f32x4 c) {
     if constexpr (BF)
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
                                                        __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
@@ -52,13 +53,13 @@ __device__ inline f32x4 mfma16(s16x8 a, s16x8 b, f32x4 c) {
 }
 
 template <bool BF>
-__device__ inline short cvt16(float x) {
+__device__ __forceinline__ short cvt16(float x) {
     if constexpr (BF) return __builtin_bit_cast(short, (__bf16)x);
     else return __builtin_bit_cast(short, (_Float16)x);
 }
 
 template <bool BF>
-__device__ inline float cvt32(short x) {
+__device__ __forceinline__ float cvt32(short x) {
     if constexpr (BF) return __uint_as_float(((uint32_t)(uint16_t)x) << 16);
     else return (float)__builtin_bit_cast(_Float16, x);
 }
@@ -66,21 +67,21 @@ __device__ inline float cvt32(short x) {
 // 4 tokens x 16 channels out of channel-major LDS, transposed: lane i of each
 // 16-lane group receives, for the channel the caller assigned to it, the values
 // of the 4 tokens addressed by lanes {i/4, 4+i/4, 8+i/4, 12+i/4}.
-__device__ inline s16x4 lds_read_tr(const short *p) {
+__device__ __forceinline__ s16x4 lds_read_tr(const short *p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
         (s16x4 __attribute__((address_space(3))) *)(p));
 }
 
-__device__ inline s16x8 cat(s16x4 lo, s16x4 hi) {
+__device__ __forceinline__ s16x8 cat(s16x4 lo, s16x4 hi) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
 // max / sum over the four lanes that share a query column (l, l^16, l^32, l^48)
-__device__ inline float col_max(float x) {
+__device__ __forceinline__ float col_max(float x) {
     x = fmaxf(x, __shfl_xor(x, 16, 64));
     return fmaxf(x, __shfl_xor(x, 32, 64));
 }
-__device__ inline float col_sum(float x) {
+__device__ __forceinline__ float col_sum(float x) {
     x += __shfl_xor(x, 16, 64);
     return x + __shfl_xor(x, 32, 64);
 }
@@ -118,7 +119,7 @@ struct Geo {
 struct Sched {
     int t, t_end, step;
 };
-__device__ inline Sched make_sched(int ntiles) {
+__device__ __forceinline__ Sched make_sched(int ntiles) {
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
     const int per = (ntiles + 7) >> 3;
     Sched sc;
@@ -131,7 +132,7 @@ __device__ inline Sched make_sched(int ntiles) {
 struct Tile {
     int bb, nn, r0, c0;
 };
-__device__ inline Tile tile_of(int t, int tiles_r, int tiles_c, int N) {
+__device__ __forceinline__ Tile tile_of(int t, int tiles_r, int tiles_c, int N) {
     Tile tl;
     tl.c0 = (t % tiles_c) * 8; t /= tiles_c;
     tl.r0 = (t % tiles_r) * 8; t /= tiles_r;
@@ -139,42 +140,72 @@ __device__ inline Tile tile_of(int t, int tiles_r, int tiles_c, int N) {
     return tl;
 }
 
-// Global -> registers: this thread's share of the halo [hr0, hr0+HR) x
-// [hc0, hc0+HC) of one image; positions at or beyond (rlim, clim) read as zero.
+// Staging plan of one thread: which 16-byte chunks of a halo it moves.  Chunk i of
+// thread t is chunk number t + 256*i of the halo in (row, column, channel-chunk)
+// order.  The plan is the same for every tile, so it is computed once.
 template <int D, int KS>
-struct HaloRegs {
-    uint4 v[Geo<D, KS>::NL];
+struct HaloPlan {
+    int rc[Geo<D, KS>::NL];  // halo row << 8 | halo column of chunk i
+    int ch8;                 // first channel of the thread's chunks
+    int lds0;                // LDS element offset of chunk 0
 };
 template <int D, int KS>
-__device__ inline void halo_fetch(HaloRegs<D, KS> &reg, const short *img, int64_t sh,
-                                  int64_t sw, int hr0, int hc0, int rlim, int clim) {
+__device__ __forceinline__ HaloPlan<D, KS> make_plan() {
     using G = Geo<D, KS>;
+    static_assert(256 % G::CPR == 0, "a thread keeps one channel chunk");
+    HaloPlan<D, KS> pl;
+    pl.ch8 = (threadIdx.x % G::CPR) * 8;
+    pl.lds0 = (threadIdx.x / G::CPR) * G::PITCH + pl.ch8;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
-        const int id = threadIdx.x + i * 256;
-        const int row = id / G::CPR, ch = id % G::CPR;
-        const int r = hr0 + row / G::HC, c = hc0 + row % G::HC;
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (id < G::NCH && r < rlim && c < clim)
-            v = *reinterpret_cast<const uint4 *>(img + r * sh + c * sw + ch * 8);
-        reg.v[i] = v;
+        int row = threadIdx.x / G::CPR + i * (256 / G::CPR);
+        row = row < G::HR * G::HC ? row : G::HR * G::HC - 1;  // tail: harmless duplicate
+        pl.rc[i] = ((row / G::HC) << 8) | (row % G::HC);
+    }
+    return pl;
+}
+template <int D, int KS>
+struct HaloRegs {
+    u32x4 v[Geo<D, KS>::NL];
+};
+// Global -> registers: this thread's share of the halo with origin (hr0, hc0) of
+// one image.  Halo positions at or beyond (rlim, clim) are not needed by any
+// unmasked product; they are clamped to the last valid row / column so the loads
+// stay in bounds and branch-free (the values only ever meet zero probabilities).
+// Addresses are a uniform base plus a 32-bit per-lane byte offset formed with
+// 24-bit multiplies: strides are below 2^22 elements (checked on the host).
+template <int D, int KS>
+__device__ __forceinline__ void halo_fetch(HaloRegs<D, KS> &reg, const HaloPlan<D, KS> &pl,
+                                  const short *img, int64_t sh, int64_t sw, int hr0, int hc0,
+                                  int rlim, int clim) {
+    using G = Geo<D, KS>;
+    const char *base = reinterpret_cast<const char *>(img + hr0 * sh + hc0 * sw);
+    const unsigned sh2 = (unsigned)sh * 2u, sw2 = (unsigned)sw * 2u;
+    const int rmax = rlim - 1 - hr0, cmax = clim - 1 - hc0;
+#pragma unroll
+    for (int i = 0; i < G::NL; i++) {
+        const unsigned r = (unsigned)min(pl.rc[i] >> 8, rmax);
+        const unsigned c = (unsigned)min(pl.rc[i] & 255, cmax);
+        const unsigned off = __umul24(r, sh2) + __umul24(c, sw2) + (unsigned)pl.ch8 * 2u;
+        reg.v[i] = *reinterpret_cast<const u32x4 *>(base + off);
     }
 }
 // Registers -> LDS, channel-major with padded pitch.
 template <int D, int KS>
-__device__ inline void halo_commit(short *lds, const HaloRegs<D, KS> &reg) {
+__device__ __forceinline__ void halo_commit(short *lds, const HaloPlan<D, KS> &pl,
+                                   const HaloRegs<D, KS> &reg) {
     using G = Geo<D, KS>;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
-        const int id = threadIdx.x + i * 256;
-        const int row = id / G::CPR, ch = id % G::CPR;
-        if (id < G::NCH) *reinterpret_cast<uint4 *>(lds + row * G::PITCH + ch * 8) = reg.v[i];
+        const int row = threadIdx.x / G::CPR + i * (256 / G::CPR);
+        if (row < G::HR * G::HC)
+            *reinterpret_cast<u32x4 *>(lds + pl.lds0 + i * (256 / G::CPR) * G::PITCH) = reg.v[i];
     }
 }
 // The spare row stays zero for the whole kernel: padding tokens and tokens
 // outside a wave's halo read it, so they add exact zeros to the second product.
 template <int D, int KS>
-__device__ inline void zero_row(short *lds) {
+__device__ __forceinline__ void zero_row(short *lds) {
     using G = Geo<D, KS>;
     if (threadIdx.x < G::CPR)
         *reinterpret_cast<uint4 *>(lds + G::ZROW * G::PITCH + threadIdx.x * 8) =
@@ -191,7 +222,7 @@ struct LaneQ {
     int64_t tok;     // flat token index of the query
 };
 template <int KS>
-__device__ inline LaneQ lane_query(const Tile &tl, const Shape &s, int wave, int n) {
+__device__ __forceinline__ LaneQ lane_query(const Tile &tl, const Shape &s, int wave, int n) {
     LaneQ q;
     const int wr0 = tl.r0 + (wave >> 1) * 4, wc0 = tl.c0 + (wave & 1) * 4;
     q.wave_on = wr0 < s.H && wc0 < s.W;
@@ -211,7 +242,7 @@ __device__ inline LaneQ lane_query(const Tile &tl, const Shape &s, int wave, int
 }
 
 template <typename T>
-__device__ inline const short *image(const View &v, const Tile &tl) {
+__device__ __forceinline__ const short *image(const View &v, const Tile &tl) {
     return static_cast<const short *>(v.ptr) + tl.bb * v.sb + tl.nn * v.sn;
 }
 
@@ -232,11 +263,12 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
     const float sc2 = s.scale * kLog2e;
 
     // registers that carry the next tile while the current one is computed
+    const HaloPlan<D, KS> plan = make_plan<D, KS>();
     HaloRegs<D, KS> kst, vst;
     s16x8 qnext[G::DS];
-    auto prefetch = [&](const Tile &tl, const LaneQ &lq) {
-        halo_fetch<D, KS>(kst, image<short>(a.k, tl), a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W);
-        halo_fetch<D, KS>(vst, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
+    auto prefetch = [&](const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
+        halo_fetch<D, KS>(kst, plan, image<short>(a.k, tl), a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W);
+        halo_fetch<D, KS>(vst, plan, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
         const short *qp = image<short>(a.q, tl) + lq.qr * a.q.sh + lq.qc * a.q.sw + g * 8;
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++)
@@ -247,8 +279,8 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
     LaneQ lq = lane_query<KS>(cur, s, wave, n);
     prefetch(cur, lq);
     for (;;) {
-        halo_commit<D, KS>(lds_k, kst);
-        halo_commit<D, KS>(lds_v, vst);
+        halo_commit<D, KS>(lds_k, plan, kst);
+        halo_commit<D, KS>(lds_v, plan, vst);
         s16x8 qreg[G::DS];
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) qreg[ds] = qnext[ds];
@@ -354,9 +386,10 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
 
 // ------------------------------------------------------------------ dQ
 // Query-centric like the forward: recompute P from the saved log-sum-exp, form
-// dP^T = V dO^T on the same halo, dS = P * (dP - delta) with delta = dO . O, and
-// dQ^T = K^T dS^T with K read back from LDS transposed.  Also writes delta for the
-// dK/dV pass.  Per-query math: e_natten/triton.py:383-398.
+// dP^T = V dO^T on the same halo, dS = P * (dP - delta) with delta = sum_j P_j dP_j
+// (equal to dO . O, so the forward output is never read), and dQ^T = K^T dS^T with
+// K read back from LDS transposed.  Also writes delta for the dK/dV pass.
+// Per-query math: e_natten/triton.py:383-398.
 template <bool BF, int D, int KS>
 __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs a, int tiles_r, int tiles_c,
                                                    int ntiles) {
@@ -373,20 +406,19 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
 
+    const HaloPlan<D, KS> plan = make_plan<D, KS>();
     HaloRegs<D, KS> kst, vst;
-    s16x8 qnext[G::DS], gnext[G::DS], onext[G::DS];
+    s16x8 qnext[G::DS], gnext[G::DS];
     float lse_next = 0.f;
-    auto prefetch = [&](const Tile &tl, const LaneQ &lq) {
-        halo_fetch<D, KS>(kst, image<short>(a.k, tl), a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W);
-        halo_fetch<D, KS>(vst, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
+    auto prefetch = [&](const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
+        halo_fetch<D, KS>(kst, plan, image<short>(a.k, tl), a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W);
+        halo_fetch<D, KS>(vst, plan, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
         const short *qp = image<short>(a.q, tl) + lq.qr * a.q.sh + lq.qc * a.q.sw + g * 8;
         const short *gp = static_cast<const short *>(a.d_o) + lq.tok * D + g * 8;
-        const short *op = static_cast<const short *>(a.o) + lq.tok * D + g * 8;
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) {
             qnext[ds] = *reinterpret_cast<const s16x8 *>(qp + ds * 32);
             gnext[ds] = *reinterpret_cast<const s16x8 *>(gp + ds * 32);
-            onext[ds] = *reinterpret_cast<const s16x8 *>(op + ds * 32);
         }
         lse_next = a.lse[lq.tok];
     };
@@ -395,17 +427,13 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
     LaneQ lq = lane_query<KS>(cur, s, wave, n);
     prefetch(cur, lq);
     for (;;) {
-        halo_commit<D, KS>(lds_k, kst);
-        halo_commit<D, KS>(lds_v, vst);
+        halo_commit<D, KS>(lds_k, plan, kst);
+        halo_commit<D, KS>(lds_v, plan, vst);
         s16x8 qreg[G::DS], greg[G::DS];
-        float dpart = 0.f;
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) {
             qreg[ds] = qnext[ds];
             greg[ds] = gnext[ds];
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-                dpart = fmaf(cvt32<BF>(gnext[ds][e]), cvt32<BF>(onext[ds][e]), dpart);
         }
         const float lse2 = lse_next * kLog2e;
         __syncthreads();
@@ -421,8 +449,10 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
         }
 
         if (lq.wave_on) {
-            const float delta = col_sum(dpart);
-            s16x8 dsb[G::KSTEPS];
+            // P^T and dP^T on the halo; delta = sum_j P_j dP_j (= dO . O) comes from
+            // the same values that form dS, so sum_j dS_j vanishes to rounding
+            f32x4 pr[G::MT], dp[G::MT];
+            float dpart = 0.f;
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
                 const int kk = mt * 16 + n;
@@ -443,10 +473,19 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
                     const int kr = tk / G::SW, kc = tk % G::SW;
                     const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
                                     (unsigned)(kc - lq.dc) < (unsigned)KS;
-                    const float p = ok ? __builtin_amdgcn_exp2f(cs[i] * sc2 - lse2) : 0.f;
-                    dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - delta));
+                    cs[i] = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - lse2 : -INFINITY);
+                    dpart = fmaf(cs[i], cp[i], dpart);
                 }
+                pr[mt] = cs;
+                dp[mt] = cp;
             }
+            const float delta = col_sum(dpart);
+            s16x8 dsb[G::KSTEPS];
+#pragma unroll
+            for (int mt = 0; mt < G::MT; mt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(pr[mt][i] * (dp[mt][i] - delta));
 
             f32x4 dq[G::DT];
 #pragma unroll
@@ -513,7 +552,7 @@ struct KeyBlock {
     bool first, last;     // first / last block of its tile
 };
 template <int KS, int HR, int HC>
-__device__ inline KeyBlock first_block(int t, int tiles_r, int tiles_c, const Shape &s) {
+__device__ __forceinline__ KeyBlock first_block(int t, int tiles_r, int tiles_c, const Shape &s) {
     KeyBlock b;
     b.t = t;
     b.tl = tile_of(t, tiles_r, tiles_c, s.N);
@@ -529,7 +568,7 @@ __device__ inline KeyBlock first_block(int t, int tiles_r, int tiles_c, const Sh
 }
 // Next block of the same tile, or false when the tile is finished.
 template <int HR, int HC>
-__device__ inline bool next_block(KeyBlock &b) {
+__device__ __forceinline__ bool next_block(KeyBlock &b) {
     if (b.last) return false;
     b.first = false;
     b.bc += HC;
@@ -558,19 +597,19 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
 
+    const HaloPlan<D, KS> plan = make_plan<D, KS>();
     HaloRegs<D, KS> qst, gst;
     float2 sst[G::NST];
-    s16x8 knext[G::DS], vnext[G::DS];
     // the wave's 4x4 keys of a tile: this lane's key pixel (clamped into the image)
-    auto key_of = [&](const Tile &tl, int &kr, int &kc) {
+    auto key_of = [&](const Tile &tl, int &kr, int &kc) __attribute__((always_inline)) {
         kr = min(tl.r0 + (wave >> 1) * 4 + (n >> 2), s.H - 1);
         kc = min(tl.c0 + (wave & 1) * 4 + (n & 3), s.W - 1);
     };
-    auto prefetch = [&](const KeyBlock &b) {
+    auto prefetch = [&](const KeyBlock &b) __attribute__((always_inline)) {
         const int64_t img_tok = ((int64_t)b.tl.bb * s.N + b.tl.nn) * s.H * (int64_t)s.W;
-        halo_fetch<D, KS>(qst, image<short>(a.q, b.tl), a.q.sh, a.q.sw, b.br, b.bc, b.qb, b.cb);
-        halo_fetch<D, KS>(gst, static_cast<const short *>(a.d_o) + img_tok * D, (int64_t)s.W * D,
-                          D, b.br, b.bc, b.qb, b.cb);
+        halo_fetch<D, KS>(qst, plan, image<short>(a.q, b.tl), a.q.sh, a.q.sw, b.br, b.bc, b.qb, b.cb);
+        halo_fetch<D, KS>(gst, plan, static_cast<const short *>(a.d_o) + img_tok * D,
+                          (int64_t)s.W * D, D, b.br, b.bc, b.qb, b.cb);
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
             const int id = threadIdx.x + i * 256;
@@ -582,37 +621,36 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
             }
             sst[i] = st;
         }
-        if (b.first) {
-            int kr, kc;
-            key_of(b.tl, kr, kc);
-            const short *kp = image<short>(a.k, b.tl) + kr * a.k.sh + kc * a.k.sw + g * 8;
-            const short *vp = image<short>(a.v, b.tl) + kr * a.v.sh + kc * a.v.sw + g * 8;
+    };
+    // B operands of the tile: this lane's key, channels ds*32 + g*8 ..  They are
+    // loaded when the previous tile's math is over and waited for after the next
+    // commit, before any newer load is issued.
+    s16x8 kreg[G::DS], vreg[G::DS];
+    auto load_keys = [&](const Tile &tl) __attribute__((always_inline)) {
+        int kr, kc;
+        key_of(tl, kr, kc);
+        const short *kp = image<short>(a.k, tl) + kr * a.k.sh + kc * a.k.sw + g * 8;
+        const short *vp = image<short>(a.v, tl) + kr * a.v.sh + kc * a.v.sw + g * 8;
 #pragma unroll
-            for (int ds = 0; ds < G::DS; ds++) {
-                knext[ds] = *reinterpret_cast<const s16x8 *>(kp + ds * 32);
-                vnext[ds] = *reinterpret_cast<const s16x8 *>(vp + ds * 32);
-            }
+        for (int ds = 0; ds < G::DS; ds++) {
+            kreg[ds] = *reinterpret_cast<const s16x8 *>(kp + ds * 32);
+            vreg[ds] = *reinterpret_cast<const s16x8 *>(vp + ds * 32);
         }
     };
 
-    s16x8 kreg[G::DS], vreg[G::DS];
     f32x4 dk[G::DT], dv[G::DT];
     KeyBlock cur = first_block<KS, G::HR, G::HC>(sc.t, tiles_r, tiles_c, s);
     prefetch(cur);
+    load_keys(cur.tl);
     for (;;) {
-        halo_commit<D, KS>(lds_q, qst);
-        halo_commit<D, KS>(lds_g, gst);
+        halo_commit<D, KS>(lds_q, plan, qst);
+        halo_commit<D, KS>(lds_g, plan, gst);
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
             const int id = threadIdx.x + i * 256;
             if (id < G::ROWS) lds_stat[id] = sst[i];
         }
         if (cur.first) {
-#pragma unroll
-            for (int ds = 0; ds < G::DS; ds++) {
-                kreg[ds] = knext[ds];
-                vreg[ds] = vnext[ds];
-            }
 #pragma unroll
             for (int mt = 0; mt < G::DT; mt++) {
                 dk[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -645,7 +683,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
             const int magic = wcols > 0 ? (65536 + wcols - 1) / wcols : 0;
             // staged row of the wave's query number qi (row-major over its rectangle);
             // qi * magic >> 16 == qi / wcols for qi < 2048, wcols <= 32
-            auto row_of = [&](int qi, int &r, int &c) {
+            auto row_of = [&](int qi, int &r, int &c) __attribute__((always_inline)) {
                 const int dvd = (qi * magic) >> 16;
                 r = ra + dvd;
                 c = cc + qi - dvd * wcols;
@@ -674,10 +712,13 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
                         const bool ok = qi < nq &&
                                         (unsigned)(kr - win_start(er, s.H, KS)) < (unsigned)KS &&
                                         (unsigned)(kc - win_start(ec, s.W, KS)) < (unsigned)KS;
-                        const float p = ok ? __builtin_amdgcn_exp2f(cs[i] * sc2 - st.x) : 0.f;
+                        const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
                         pb[m2 * 4 + i] = cvt16<BF>(p);
                         dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
                     }
+                    // keep the second half's operand loads from being hoisted above
+                    // the first half: the register budget has no room for both
+                    __builtin_amdgcn_sched_barrier(0);
                 }
                 const short *qt[2], *gt[2];
 #pragma unroll
@@ -719,6 +760,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
         }
 
         if (!more) break;
+        if (nxt.first) load_keys(nxt.tl);
         __syncthreads();
         cur = nxt;
     }
@@ -741,7 +783,7 @@ int check_launch(const char *what) {
 
 bool layout_ok(const View &v) {
     return reinterpret_cast<uintptr_t>(v.ptr) % 16 == 0 && v.sb % 8 == 0 && v.sn % 8 == 0 &&
-           v.sh % 8 == 0 && v.sw % 8 == 0;
+           v.sh % 8 == 0 && v.sw % 8 == 0 && v.sh < (1 << 22) && v.sw < (1 << 22);
 }
 
 // Persistent grid: as many workgroups as stay resident at once (8 XCDs x 32 CUs x
