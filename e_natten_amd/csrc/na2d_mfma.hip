@@ -551,21 +551,6 @@ struct KeyBlock {
     int br, bc;           // origin of the staged block of queries
     bool first, last;     // first / last block of its tile
 };
-template <int KS, int HR, int HC>
-__device__ __forceinline__ KeyBlock first_block(int t, int tiles_r, int tiles_c, const Shape &s) {
-    KeyBlock b;
-    b.t = t;
-    b.tl = tile_of(t, tiles_r, tiles_c, s.N);
-    b.qa = inv_lo(b.tl.r0, KS);
-    b.qb = inv_hi(min(b.tl.r0 + 8, s.H) - 1, s.H, KS);
-    b.ca = inv_lo(b.tl.c0, KS);
-    b.cb = inv_hi(min(b.tl.c0 + 8, s.W) - 1, s.W, KS);
-    b.br = b.qa;
-    b.bc = b.ca;
-    b.first = true;
-    b.last = b.br + HR >= b.qb && b.bc + HC >= b.cb;
-    return b;
-}
 // Next block of the same tile, or false when the tile is finished.
 template <int HR, int HC>
 __device__ __forceinline__ bool next_block(KeyBlock &b) {
@@ -580,9 +565,207 @@ __device__ __forceinline__ bool next_block(KeyBlock &b) {
     return true;
 }
 
+// The tiles of an image split into an inner rectangle, where no key or query is
+// within reach of the border, and the frame around it.
+struct TileSet {
+    int tiles_r, tiles_c;  // 8x8 tiles per image
+    int ir0, ni_r;         // first inner tile row, number of inner tile rows
+    int ic0, ni_c;         // first inner tile column, number of inner tile columns
+};
+__device__ __forceinline__ Tile inner_tile(int t, const TileSet &ts, int N) {
+    Tile tl;
+    tl.c0 = (ts.ic0 + t % ts.ni_c) * 8; t /= ts.ni_c;
+    tl.r0 = (ts.ir0 + t % ts.ni_r) * 8; t /= ts.ni_r;
+    tl.bb = t / N; tl.nn = t % N;
+    return tl;
+}
+__device__ __forceinline__ Tile frame_tile(int t, const TileSet &ts, int N) {
+    const int per_img = ts.tiles_r * ts.tiles_c - ts.ni_r * ts.ni_c;
+    const int slab = t / per_img;
+    int e = t % per_img;
+    const int top = ts.ir0 * ts.tiles_c, side = ts.tiles_c - ts.ni_c;
+    int tr, tc;
+    if (e < top) {
+        tr = e / ts.tiles_c; tc = e % ts.tiles_c;
+    } else if (e < top + ts.ni_r * side) {
+        e -= top;
+        tr = ts.ir0 + e / side;
+        tc = e % side;
+        tc = tc < ts.ic0 ? tc : tc + ts.ni_c;
+    } else {
+        e -= top + ts.ni_r * side;
+        tr = ts.ir0 + ts.ni_r + e / ts.tiles_c; tc = e % ts.tiles_c;
+    }
+    Tile tl;
+    tl.r0 = tr * 8; tl.c0 = tc * 8;
+    tl.bb = slab / N; tl.nn = slab % N;
+    return tl;
+}
+
+// Inner tiles.  Every key is attended by exactly the queries within k//2 of it
+// and all windows are centred, so the picture is the forward's with the roles of
+// queries and keys exchanged: the staged block is the tile's (8+k-1)^2 halo of
+// queries, a wave's queries are the (4+k-1)^2 halo of its 4x4 keys at a fixed
+// place in it, and the mask depends on the lane only.
 template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArgs a, int tiles_r, int tiles_c,
-                                                     int ntiles) {
+__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_inner_mfma(BwdArgs a,
+                                                                              TileSet ts,
+                                                                              int ntiles) {
+    using G = Geo<D, KS>;
+    __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
+    __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
+    __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
+
+    const Shape &s = a.s;
+    Sched sc = make_sched(ntiles);
+    if (sc.t >= sc.t_end) return;
+    zero_row<D, KS>(lds_q);
+    zero_row<D, KS>(lds_g);
+    if (threadIdx.x == 0) lds_stat[G::ZROW] = make_float2(0.f, 0.f);
+
+    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const float sc2 = s.scale * kLog2e;
+    const int orow = (wave >> 1) * 4, ocol = (wave & 1) * 4;
+    auto row_of = [&](int tk) __attribute__((always_inline)) {
+        return tk < G::NK ? (orow + tk / G::SW) * G::HC + ocol + tk % G::SW : (int)G::ZROW;
+    };
+
+    const HaloPlan<D, KS> plan = make_plan<D, KS>();
+    HaloRegs<D, KS> qst, gst;
+    float2 sst[G::NST];
+    auto prefetch = [&](const Tile &tl) __attribute__((always_inline)) {
+        const int64_t img_tok = ((int64_t)tl.bb * s.N + tl.nn) * s.H * (int64_t)s.W;
+        const int br = tl.r0 - KS / 2, bc = tl.c0 - KS / 2;
+        halo_fetch<D, KS>(qst, plan, image<short>(a.q, tl), a.q.sh, a.q.sw, br, bc, s.H, s.W);
+        halo_fetch<D, KS>(gst, plan, static_cast<const short *>(a.d_o) + img_tok * D,
+                          (int64_t)s.W * D, D, br, bc, s.H, s.W);
+#pragma unroll
+        for (int i = 0; i < G::NST; i++) {
+            const int id = min((int)threadIdx.x + i * 256, G::ZROW - 1);
+            const int64_t qt = img_tok + (int64_t)(br + id / G::HC) * s.W + bc + id % G::HC;
+            sst[i] = make_float2(a.lse[qt] * kLog2e, a.delta[qt]);
+        }
+    };
+    // B operands of a tile: this lane's key, channels ds*32 + g*8 ..  Loaded when
+    // the previous tile's math is over (they would not fit beside it) and complete
+    // before the barrier below, i.e. before any newer load is in flight.
+    s16x8 kreg[G::DS], vreg[G::DS];
+    auto load_keys = [&](const Tile &tl) __attribute__((always_inline)) {
+        const int kr = tl.r0 + orow + (n >> 2), kc = tl.c0 + ocol + (n & 3);
+        const short *kp = image<short>(a.k, tl) + kr * a.k.sh + kc * a.k.sw + g * 8;
+        const short *vp = image<short>(a.v, tl) + kr * a.v.sh + kc * a.v.sw + g * 8;
+#pragma unroll
+        for (int ds = 0; ds < G::DS; ds++) {
+            kreg[ds] = *reinterpret_cast<const s16x8 *>(kp + ds * 32);
+            vreg[ds] = *reinterpret_cast<const s16x8 *>(vp + ds * 32);
+        }
+    };
+
+    Tile cur = inner_tile(sc.t, ts, s.N);
+    prefetch(cur);
+    load_keys(cur);
+    for (;;) {
+        halo_commit<D, KS>(lds_q, plan, qst);
+        halo_commit<D, KS>(lds_g, plan, gst);
+#pragma unroll
+        for (int i = 0; i < G::NST; i++) {
+            const int id = threadIdx.x + i * 256;
+            if (id < G::ZROW) lds_stat[id] = sst[i];
+        }
+#pragma unroll
+        for (int ds = 0; ds < G::DS; ds++) asm volatile("" : "+v"(kreg[ds]), "+v"(vreg[ds]));
+        __syncthreads();
+
+        const int tn = sc.t + sc.step;
+        const bool more = tn < sc.t_end;
+        Tile nxt = cur;
+        if (more) {
+            nxt = inner_tile(tn, ts, s.N);
+            prefetch(nxt);
+        }
+
+        f32x4 dk[G::DT], dv[G::DT];
+#pragma unroll
+        for (int mt = 0; mt < G::DT; mt++) {
+            dk[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            dv[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int ks = 0; ks < G::KSTEPS; ks++) {
+            s16x8 pb, dsb;
+#pragma unroll
+            for (int m2 = 0; m2 < 2; m2++) {
+                const int mt = ks * 2 + m2;
+                const int row = row_of(mt * 16 + n);
+                const short *qp = lds_q + row * G::PITCH + g * 8;
+                const short *gp = lds_g + row * G::PITCH + g * 8;
+                f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ds = 0; ds < G::DS; ds++) {
+                    cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32), kreg[ds], cs);
+                    cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32), vreg[ds], cp);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int tk = mt * 16 + g * 4 + i;  // query of accumulator row g*4+i
+                    const float2 st = lds_stat[row_of(tk)];
+                    const bool ok = tk < G::NK &&
+                                    (unsigned)(tk / G::SW - (n >> 2)) < (unsigned)KS &&
+                                    (unsigned)(tk % G::SW - (n & 3)) < (unsigned)KS;
+                    const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
+                    pb[m2 * 4 + i] = cvt16<BF>(p);
+                    dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
+                }
+            }
+            const short *qt[2], *gt[2];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int row = row_of(ks * 32 + h * 16 + g * 4 + (n >> 2));
+                qt[h] = lds_q + row * G::PITCH + (n & 3) * (D / 4);
+                gt[h] = lds_g + row * G::PITCH + (n & 3) * (D / 4);
+            }
+#pragma unroll
+            for (int mt = 0; mt < G::DT; mt++) {
+                dv[mt] = mfma16<BF>(cat(lds_read_tr(gt[0] + mt * 4), lds_read_tr(gt[1] + mt * 4)),
+                                    pb, dv[mt]);
+                dk[mt] = mfma16<BF>(cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)),
+                                    dsb, dk[mt]);
+            }
+        }
+
+        {
+            const int kr = cur.r0 + orow + (n >> 2), kc = cur.c0 + ocol + (n & 3);
+            const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + kr) * s.W + kc;
+            short *dkp = static_cast<short *>(a.dk) + tok * D + g * (D / 4);
+            short *dvp = static_cast<short *>(a.dv) + tok * D + g * (D / 4);
+#pragma unroll
+            for (int j = 0; j < G::DT / 2; j++) {
+                s16x8 wk, wv;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    wk[i] = cvt16<BF>(dk[2 * j][i] * s.scale);
+                    wk[4 + i] = cvt16<BF>(dk[2 * j + 1][i] * s.scale);
+                    wv[i] = cvt16<BF>(dv[2 * j][i]);
+                    wv[4 + i] = cvt16<BF>(dv[2 * j + 1][i]);
+                }
+                *reinterpret_cast<s16x8 *>(dkp + j * 8) = wk;
+                *reinterpret_cast<s16x8 *>(dvp + j * 8) = wv;
+            }
+        }
+
+        if (!more) break;
+        load_keys(nxt);
+        __syncthreads();
+        cur = nxt;
+        sc.t = tn;
+    }
+}
+
+// Frame tiles: the general case, walked block by block (see above).
+template <bool BF, int D, int KS>
+__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_frame_mfma(BwdArgs a,
+                                                                              TileSet ts,
+                                                                              int ntiles) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
@@ -605,7 +788,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
         kr = min(tl.r0 + (wave >> 1) * 4 + (n >> 2), s.H - 1);
         kc = min(tl.c0 + (wave & 1) * 4 + (n & 3), s.W - 1);
     };
-    auto prefetch = [&](const KeyBlock &b) __attribute__((always_inline)) {
+    auto stage = [&](const KeyBlock &b) __attribute__((always_inline)) {
         const int64_t img_tok = ((int64_t)b.tl.bb * s.N + b.tl.nn) * s.H * (int64_t)s.W;
         halo_fetch<D, KS>(qst, plan, image<short>(a.q, b.tl), a.q.sh, a.q.sw, b.br, b.bc, b.qb, b.cb);
         halo_fetch<D, KS>(gst, plan, static_cast<const short *>(a.d_o) + img_tok * D,
@@ -613,18 +796,12 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
             const int id = threadIdx.x + i * 256;
-            const int r = b.br + id / G::HC, c = b.bc + id % G::HC;
-            float2 st = make_float2(0.f, 0.f);
-            if (id < G::ZROW && r < b.qb && c < b.cb) {
-                const int64_t qt = img_tok + (int64_t)r * s.W + c;
-                st = make_float2(a.lse[qt] * kLog2e, a.delta[qt]);
-            }
-            sst[i] = st;
+            const int r = min(b.br + id / G::HC, b.qb - 1), c = min(b.bc + id % G::HC, b.cb - 1);
+            const int64_t qt = img_tok + (int64_t)r * s.W + c;
+            sst[i] = make_float2(a.lse[qt] * kLog2e, a.delta[qt]);
         }
     };
-    // B operands of the tile: this lane's key, channels ds*32 + g*8 ..  They are
-    // loaded when the previous tile's math is over and waited for after the next
-    // commit, before any newer load is issued.
+    // B operands of the tile: this lane's key, channels ds*32 + g*8 ..
     s16x8 kreg[G::DS], vreg[G::DS];
     auto load_keys = [&](const Tile &tl) __attribute__((always_inline)) {
         int kr, kc;
@@ -637,10 +814,28 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
             vreg[ds] = *reinterpret_cast<const s16x8 *>(vp + ds * 32);
         }
     };
+    auto first_of = [&](int t) __attribute__((always_inline)) {
+        KeyBlock b;
+        b.t = t;
+        b.tl = frame_tile(t, ts, s.N);
+        b.qa = inv_lo(b.tl.r0, KS);
+        b.qb = inv_hi(min(b.tl.r0 + 8, s.H) - 1, s.H, KS);
+        b.ca = inv_lo(b.tl.c0, KS);
+        b.cb = inv_hi(min(b.tl.c0 + 8, s.W) - 1, s.W, KS);
+        b.br = b.qa;
+        b.bc = b.ca;
+        b.first = true;
+        b.last = b.br + G::HR >= b.qb && b.bc + G::HC >= b.cb;
+        return b;
+    };
 
     f32x4 dk[G::DT], dv[G::DT];
-    KeyBlock cur = first_block<KS, G::HR, G::HC>(sc.t, tiles_r, tiles_c, s);
-    prefetch(cur);
+    KeyBlock cur = first_of(sc.t);
+    // The loads of a block are issued when the previous block's math is over; the
+    // other workgroup on the CU covers their latency.  (These tiles are the
+    // minority; keeping the loads in flight across the math would need registers
+    // that the two accumulators do not leave.)
+    stage(cur);
     load_keys(cur.tl);
     for (;;) {
         halo_commit<D, KS>(lds_q, plan, qst);
@@ -648,7 +843,8 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
             const int id = threadIdx.x + i * 256;
-            if (id < G::ROWS) lds_stat[id] = sst[i];
+            if (id < G::ZROW) lds_stat[id] = sst[i];
+            else if (id == G::ZROW) lds_stat[id] = make_float2(0.f, 0.f);
         }
         if (cur.first) {
 #pragma unroll
@@ -662,39 +858,35 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
         KeyBlock nxt = cur;
         bool more = next_block<G::HR, G::HC>(nxt);
         if (!more && cur.t + sc.step < sc.t_end) {
-            nxt = first_block<KS, G::HR, G::HC>(cur.t + sc.step, tiles_r, tiles_c, s);
+            nxt = first_of(cur.t + sc.step);
             more = true;
         }
-        if (more) prefetch(nxt);
-
         const int wr0 = cur.tl.r0 + (wave >> 1) * 4, wc0 = cur.tl.c0 + (wave & 1) * 4;
         const bool wave_on = wr0 < s.H && wc0 < s.W;
         int kr, kc;
         key_of(cur.tl, kr, kc);
         if (wave_on) {
             // this wave's queries inside the staged block: those that attend to any
-            // of its 4x4 keys
+            // of its 4x4 keys, numbered row-major over their rectangle
             const int ra = max(inv_lo(wr0, KS), cur.br);
             const int rb = min(inv_hi(min(wr0 + 4, s.H) - 1, s.H, KS), cur.br + G::HR);
             const int cc = max(inv_lo(wc0, KS), cur.bc);
             const int cd = min(inv_hi(min(wc0 + 4, s.W) - 1, s.W, KS), cur.bc + G::HC);
             const int wcols = cd - cc;
             const int nq = (rb > ra && cd > cc) ? (rb - ra) * wcols : 0;
-            const int magic = wcols > 0 ? (65536 + wcols - 1) / wcols : 0;
-            // staged row of the wave's query number qi (row-major over its rectangle);
             // qi * magic >> 16 == qi / wcols for qi < 2048, wcols <= 32
-            auto row_of = [&](int qi, int &r, int &c) __attribute__((always_inline)) {
+            const int magic = wcols > 0 ? (65536 + wcols - 1) / wcols : 0;
+            // staged row of query qi (zero row past the end), branch-free
+            auto row_of = [&](int qi) __attribute__((always_inline)) {
                 const int dvd = (qi * magic) >> 16;
-                r = ra + dvd;
-                c = cc + qi - dvd * wcols;
-                return qi < nq ? (r - cur.br) * G::HC + (c - cur.bc) : (int)G::ZROW;
+                const int row = (ra + dvd - cur.br) * G::HC + (cc + qi - dvd * wcols - cur.bc);
+                return qi < nq ? row : (int)G::ZROW;
             };
             for (int q0 = 0; q0 < nq; q0 += 32) {
                 s16x8 pb, dsb;
 #pragma unroll
                 for (int m2 = 0; m2 < 2; m2++) {
-                    int rr, rc;
-                    const int row = row_of(q0 + m2 * 16 + n, rr, rc);
+                    const int row = row_of(q0 + m2 * 16 + n);
                     const short *qp = lds_q + row * G::PITCH + g * 8;
                     const short *gp = lds_g + row * G::PITCH + g * 8;
                     f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
@@ -706,25 +898,23 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         const int qi = q0 + m2 * 16 + g * 4 + i;
-                        int er, ec;
-                        const int erow = row_of(qi, er, ec);
-                        const float2 st = lds_stat[erow];
-                        const bool ok = qi < nq &&
-                                        (unsigned)(kr - win_start(er, s.H, KS)) < (unsigned)KS &&
-                                        (unsigned)(kc - win_start(ec, s.W, KS)) < (unsigned)KS;
-                        const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
+                        const int dvd = (qi * magic) >> 16;
+                        const int er = ra + dvd, ec = cc + qi - dvd * wcols;
+                        const float2 st = lds_stat[row_of(qi)];
+                        const bool ok =
+                            (qi < nq) &
+                            ((unsigned)(kr - win_start(er, s.H, KS)) < (unsigned)KS) &
+                            ((unsigned)(kc - win_start(ec, s.W, KS)) < (unsigned)KS);
+                        const float p =
+                            __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
                         pb[m2 * 4 + i] = cvt16<BF>(p);
                         dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
                     }
-                    // keep the second half's operand loads from being hoisted above
-                    // the first half: the register budget has no room for both
-                    __builtin_amdgcn_sched_barrier(0);
                 }
                 const short *qt[2], *gt[2];
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
-                    int rr, rc;
-                    const int row = row_of(q0 + h * 16 + g * 4 + (n >> 2), rr, rc);
+                    const int row = row_of(q0 + h * 16 + g * 4 + (n >> 2));
                     qt[h] = lds_q + row * G::PITCH + (n & 3) * (D / 4);
                     gt[h] = lds_g + row * G::PITCH + (n & 3) * (D / 4);
                 }
@@ -760,6 +950,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
         }
 
         if (!more) break;
+        stage(nxt);
         if (nxt.first) load_keys(nxt.tl);
         __syncthreads();
         cur = nxt;
@@ -830,11 +1021,27 @@ int bwd_launch(const BwdArgs &a, hipStream_t st) {
             hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
                                tiles_c, (int)nb);
         }
-        {
-            const int grid = persistent_grid(bwd_dkdv_mfma<BF, D, KS>, nb);
-            ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
-            hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
-                               tiles_c, (int)nb);
+        // dK/dV: inner tiles (no key or query within reach of the border) and frame
+        TileSet ts;
+        ts.tiles_r = tiles_r; ts.tiles_c = tiles_c;
+        ts.ir0 = (KS + 7) / 8; ts.ic0 = (KS + 7) / 8;
+        ts.ni_r = (a.s.H - KS) / 8 - ts.ir0; ts.ni_c = (a.s.W - KS) / 8 - ts.ic0;
+        if (ts.ni_r <= 0 || ts.ni_c <= 0) {
+            ts.ir0 = tiles_r; ts.ic0 = 0; ts.ni_r = 0; ts.ni_c = 0;
+        }
+        const int64_t slabs = (int64_t)a.s.B * a.s.N;
+        const int64_t n_inner = slabs * ts.ni_r * ts.ni_c, n_frame = nb - n_inner;
+        if (n_inner > 0) {
+            const int grid = persistent_grid(bwd_dkdv_inner_mfma<BF, D, KS>, n_inner);
+            ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_inner_mfma", st);
+            hipLaunchKernelGGL((bwd_dkdv_inner_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a,
+                               ts, (int)n_inner);
+        }
+        if (n_frame > 0) {
+            const int grid = persistent_grid(bwd_dkdv_frame_mfma<BF, D, KS>, n_frame);
+            ProfScope prof(ENATTEN_KERNEL_BWD_DKDV_FRAME, "bwd_dkdv_frame_mfma", st);
+            hipLaunchKernelGGL((bwd_dkdv_frame_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a,
+                               ts, (int)n_frame);
         }
         return check_launch("enatten2d_bwd");
     } else {
