@@ -175,7 +175,7 @@ def main():
     names = list(kern)
     dom = max(names, key=lambda n: kern[n]["avg_us"])
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
     if os.path.exists(tpath):
         rec = json.load(open(tpath)).get("%s/side%d/%s" % (kern[dom]["kernel"], S, args.dtype))
         traffic = rec["bytes_per_launch"] if rec else None
