@@ -27,6 +27,9 @@ SIGNATURES = {
     "enatten2d_fwd": (_i, [_vp] * 5 + [_i] * 7 + [_sp] * 3 + [ctypes.c_float, _vp]),
     "enatten2d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 4),
     "enatten2d_bwd": (_i, [_vp] * 10 + [_i] * 7 + [_sp] * 3 + [ctypes.c_float, _vp]),
+    "enatten1d_fwd": (_i, [_vp] * 5 + [_i] * 6 + [_sp] * 3 + [ctypes.c_float, _vp]),
+    "enatten1d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 3),
+    "enatten1d_bwd": (_i, [_vp] * 10 + [_i] * 6 + [_sp] * 3 + [ctypes.c_float, _vp]),
     "enatten_profile_enable": (_i, [_i]),
     "enatten_profile_read": (_i, [_i, ctypes.POINTER(_i), ctypes.POINTER(ctypes.c_double)]),
     "enatten_profile_kernel_name": (ctypes.c_char_p, [_i]),
@@ -56,6 +59,11 @@ def load() -> ctypes.CDLL:
 
 def last_error() -> str:
     return load().enatten_last_error().decode()
+
+
+def strides3(t) -> ctypes.Array:
+    """Element strides of the (batch, head, position) axes as int64_t[3]."""
+    return (ctypes.c_int64 * 3)(*t.stride()[:3])
 
 
 def strides4(t) -> ctypes.Array:

@@ -194,6 +194,85 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o, co
     return launch_bwd_simt(a, dtype, st);
 }
 
+static int view_1d(const char *fn, const char *name, const void *p, const int64_t *st, int N,
+                   int T, int D, View *out) {
+    if (!p) {
+        set_error("%s: %s is NULL", fn, name);
+        return ENATTEN_EINVAL;
+    }
+    out->ptr = p;
+    out->sh = 0;
+    if (st) {
+        out->sb = st[0]; out->sn = st[1]; out->sw = st[2];
+        if (out->sb < 0 || out->sn < 0 || out->sw < 0) {
+            set_error("%s: negative stride for %s", fn, name);
+            return ENATTEN_EINVAL;
+        }
+    } else {
+        out->sw = D;
+        out->sn = (int64_t)T * D;
+        out->sb = (int64_t)N * T * D;
+    }
+    return ENATTEN_OK;
+}
+
+static int check_shape_1d(const char *fn, int B, int N, int T, int D, int ks, int dtype) {
+    if (ks >= 1 && ks % 2 == 1 && T >= 1 && T < ks) {
+        set_error("%s: sequence length %d is smaller than kernel_size %d", fn, T, ks);
+        return ENATTEN_EINVAL;
+    }
+    return check_shape(fn, B, N, T, T, D, ks, dtype);
+}
+
+int enatten1d_fwd(const void *q, const void *k, const void *v, void *o, float *lse, int B,
+                  int heads, int T, int D, int kernel_size, int dtype, const int64_t *q_strides,
+                  const int64_t *k_strides, const int64_t *v_strides, float scale,
+                  void *stream) {
+    const char *fn = "enatten1d_fwd";
+    int rc = check_shape_1d(fn, B, heads, T, D, kernel_size, dtype);
+    if (rc) return rc;
+    FwdArgs a;
+    if ((rc = view_1d(fn, "q", q, q_strides, heads, T, D, &a.q))) return rc;
+    if ((rc = view_1d(fn, "k", k, k_strides, heads, T, D, &a.k))) return rc;
+    if ((rc = view_1d(fn, "v", v, v_strides, heads, T, D, &a.v))) return rc;
+    if (!o) {
+        set_error("%s: o is NULL", fn);
+        return ENATTEN_EINVAL;
+    }
+    a.o = o;
+    a.lse = lse;
+    a.s = Shape{B, heads, 1, T, D, 1, kernel_size, scale};  // a 1 x k window on a 1 x T image
+    return launch_fwd_simt(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+size_t enatten1d_bwd_workspace_bytes(int B, int heads, int T) {
+    return enatten2d_bwd_workspace_bytes(B, heads, 1, T);
+}
+
+int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                  const float *lse, void *dq, void *dk, void *dv, void *workspace, int B,
+                  int heads, int T, int D, int kernel_size, int dtype, const int64_t *q_strides,
+                  const int64_t *k_strides, const int64_t *v_strides, float scale,
+                  void *stream) {
+    const char *fn = "enatten1d_bwd";
+    int rc = check_shape_1d(fn, B, heads, T, D, kernel_size, dtype);
+    if (rc) return rc;
+    BwdArgs a;
+    if ((rc = view_1d(fn, "q", q, q_strides, heads, T, D, &a.q))) return rc;
+    if ((rc = view_1d(fn, "k", k, k_strides, heads, T, D, &a.k))) return rc;
+    if ((rc = view_1d(fn, "v", v, v_strides, heads, T, D, &a.v))) return rc;
+    if (!o || !d_o || !lse || !dq || !dk || !dv || !workspace) {
+        set_error("%s: o, d_o, lse, dq, dk, dv and workspace must all be non-NULL", fn);
+        return ENATTEN_EINVAL;
+    }
+    a.o = o; a.d_o = d_o; a.lse = lse;
+    a.dq = dq; a.dk = dk; a.dv = dv;
+    a.delta = static_cast<float *>(workspace);
+    a.zinv = a.delta + (size_t)B * heads * T;
+    a.s = Shape{B, heads, 1, T, D, 1, kernel_size, scale};
+    return launch_bwd_simt(a, dtype, static_cast<hipStream_t>(stream));
+}
+
 int enatten_profile_enable(int on) {
     const int prev = g_prof_on ? 1 : 0;
     if (on)

@@ -104,7 +104,8 @@ constexpr int tile_w(int qpw) {
 }
 
 // Position of this lane group's pixel: workgroups tile each (batch, head) image
-// with TH x TW blocks of pixels.
+// with TH x TW blocks of pixels, or with runs of TH*TW positions when the image
+// has a single row (the 1D operator).
 template <int G>
 struct Place {
     static constexpr int QPW = 256 / G;
@@ -120,8 +121,13 @@ struct Place {
         b = slab / s.N; n = slab % s.N;
         const int qi = threadIdx.x / G;
         lg = threadIdx.x % G;
-        x = tx * TH + qi / TW;
-        y = ty * TW + qi % TW;
+        if (s.H == 1) {
+            x = 0;
+            y = ty * QPW + qi;
+        } else {
+            x = tx * TH + qi / TW;
+            y = ty * TW + qi % TW;
+        }
         live = x < s.H && y < s.W;
         x = min(x, s.H - 1);
         y = min(y, s.W - 1);
@@ -366,8 +372,13 @@ int check_launch(const char *what) {
 
 template <int G>
 dim3 grid_for(const Shape &s, int &tiles_x, int &tiles_y) {
-    tiles_x = (s.H + Place<G>::TH - 1) / Place<G>::TH;
-    tiles_y = (s.W + Place<G>::TW - 1) / Place<G>::TW;
+    if (s.H == 1) {
+        tiles_x = 1;
+        tiles_y = (s.W + Place<G>::QPW - 1) / Place<G>::QPW;
+    } else {
+        tiles_x = (s.H + Place<G>::TH - 1) / Place<G>::TH;
+        tiles_y = (s.W + Place<G>::TW - 1) / Place<G>::TW;
+    }
     return dim3((unsigned)((int64_t)s.B * s.N * tiles_x * tiles_y));
 }
 

@@ -17,12 +17,14 @@ from . import _lib
 _DTYPES = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
 
 
-def _validate(q, k, v, kernel_size: int) -> None:
+def _validate(q, k, v, kernel_size: int, ndim: int = 5) -> None:
     for name, t in (("q", q), ("k", k), ("v", v)):
         if not isinstance(t, torch.Tensor):
             raise TypeError("%s must be a tensor" % name)
-    if q.dim() != 5:
-        raise ValueError("expected [B, heads, H, W, head_dim] tensors, got %d-D q" % q.dim())
+    if q.dim() != ndim:
+        raise ValueError("expected %s tensors, got %d-D q"
+                         % ("[B, heads, H, W, head_dim]" if ndim == 5 else "[B, heads, T, head_dim]",
+                            q.dim()))
     if k.shape != q.shape or v.shape != q.shape:
         raise ValueError("q, k and v must have the same shape, got %s, %s, %s"
                          % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
@@ -36,19 +38,19 @@ def _validate(q, k, v, kernel_size: int) -> None:
         raise TypeError("kernel_size must be an int")
     if kernel_size < 1 or kernel_size % 2 == 0:
         raise ValueError("kernel_size must be odd and >= 1, got %d" % kernel_size)
-    if q.shape[2] < kernel_size or q.shape[3] < kernel_size:
-        raise ValueError("image %dx%d is smaller than kernel_size %d"
-                         % (q.shape[2], q.shape[3], kernel_size))
+    if any(side < kernel_size for side in q.shape[2:-1]):
+        raise ValueError("input of extent %s is smaller than kernel_size %d"
+                         % ("x".join(str(x) for x in q.shape[2:-1]), kernel_size))
     if q.numel() == 0:
         raise ValueError("empty tensors are not supported")
-    if q.shape[4] > 1024:
-        raise ValueError("head_dim %d exceeds the supported maximum of 1024" % q.shape[4])
+    if q.shape[-1] > 1024:
+        raise ValueError("head_dim %d exceeds the supported maximum of 1024" % q.shape[-1])
 
 
 def _kernel_layout(t: torch.Tensor) -> torch.Tensor:
-    """The kernels take any (batch, head, row, column) strides but need unit
-    stride on the channel axis and no negative strides."""
-    if t.stride(4) != 1 and t.shape[4] != 1:
+    """The kernels take any strides on the leading axes but need unit stride on
+    the channel axis and no negative strides."""
+    if t.stride(-1) != 1 and t.shape[-1] != 1:
         return t.contiguous()
     return t
 
@@ -106,6 +108,48 @@ def _bwd_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
     return dq, dk, dv
 
 
+def _fwd1d_impl(q, k, v, kernel_size: int, scale: float):
+    _validate(q, k, v, kernel_size, 4)
+    _require_gpu(q, "enatten::na1d_fwd")
+    lib = _lib.load()
+    q, k, v = (_kernel_layout(t) for t in (q, k, v))
+    B, N, T, D = q.shape
+    o = torch.empty((B, N, T, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, N, T), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(lib.enatten1d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                 lse.data_ptr(), B, N, T, D, kernel_size, _DTYPES[q.dtype],
+                                 _lib.strides3(q), _lib.strides3(k), _lib.strides3(v),
+                                 float(scale), stream))
+    return o, lse
+
+
+def _bwd1d_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
+    _validate(q, k, v, kernel_size, 4)
+    _require_gpu(q, "enatten::na1d_bwd")
+    if d_o.shape != q.shape or o.shape != q.shape:
+        raise ValueError("o and d_o must have the shape of q")
+    if d_o.dtype != q.dtype or o.dtype != q.dtype:
+        raise ValueError("o and d_o must have the dtype of q")
+    lib = _lib.load()
+    q, k, v = (_kernel_layout(t) for t in (q, k, v))
+    o, d_o, lse = o.contiguous(), d_o.contiguous(), lse.contiguous()
+    B, N, T, D = q.shape
+    dq = torch.empty((B, N, T, D), dtype=q.dtype, device=q.device)
+    dk, dv = torch.empty_like(dq), torch.empty_like(dq)
+    ws = torch.empty(lib.enatten1d_bwd_workspace_bytes(B, N, T), dtype=torch.uint8,
+                     device=q.device)
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(lib.enatten1d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                 d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                 dv.data_ptr(), ws.data_ptr(), B, N, T, D, kernel_size,
+                                 _DTYPES[q.dtype], _lib.strides3(q), _lib.strides3(k),
+                                 _lib.strides3(v), float(scale), stream))
+    return dq, dk, dv
+
+
 # torch custom ops: thin shims over the C ABI
 _torch_lib = torch.library.Library("enatten", "DEF")
 _torch_lib.define("na2d_fwd(Tensor q, Tensor k, Tensor v, int kernel_size, float scale) "
@@ -114,6 +158,12 @@ _torch_lib.define("na2d_bwd(Tensor q, Tensor k, Tensor v, Tensor o, Tensor lse, 
                   "int kernel_size, float scale) -> (Tensor, Tensor, Tensor)")
 _torch_lib.impl("na2d_fwd", _fwd_impl, "CompositeExplicitAutograd")
 _torch_lib.impl("na2d_bwd", _bwd_impl, "CompositeExplicitAutograd")
+_torch_lib.define("na1d_fwd(Tensor q, Tensor k, Tensor v, int kernel_size, float scale) "
+                  "-> (Tensor, Tensor)")
+_torch_lib.define("na1d_bwd(Tensor q, Tensor k, Tensor v, Tensor o, Tensor lse, Tensor d_o, "
+                  "int kernel_size, float scale) -> (Tensor, Tensor, Tensor)")
+_torch_lib.impl("na1d_fwd", _fwd1d_impl, "CompositeExplicitAutograd")
+_torch_lib.impl("na1d_bwd", _bwd1d_impl, "CompositeExplicitAutograd")
 
 
 class Natten2d(torch.autograd.Function):
@@ -146,6 +196,31 @@ class Natten2d(torch.autograd.Function):
 
 
 natten2d = Natten2d.apply
+
+
+class Natten1d(torch.autograd.Function):
+    """1D neighborhood attention, ``[B, heads, T, d]`` in and out; same contract
+    as the reference Function (e_natten/triton.py:425-483)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, kernel_size=7, scale=1.0):
+        _validate(q, k, v, kernel_size, 4)
+        o, lse = torch.ops.enatten.na1d_fwd(q, k, v, kernel_size, scale)
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.kernel_size = kernel_size
+        ctx.scale = scale
+        return o
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_output):
+        q, k, v, o, lse = ctx.saved_tensors
+        dQ, dK, dV = torch.ops.enatten.na1d_bwd(q, k, v, o, lse, grad_output,
+                                                 ctx.kernel_size, ctx.scale)
+        return dQ, dK, dV, None, None
+
+
+natten1d = Natten1d.apply
 
 
 def kernel_path(head_dim: int, kernel_size: int, dtype: torch.dtype) -> str:

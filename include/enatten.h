@@ -101,6 +101,25 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o,
                   void *stream);
 
 /*
+ * 1D neighborhood attention on [B, heads, T, D] tensors: query t attends the
+ * kernel_size keys starting at clamp(t - kernel_size/2, 0, T - kernel_size).
+ * Replace the launches of _attn_fwd_1d / _attn_bwd_1d in Natten1d
+ * (e_natten/triton.py:444-450, :472-481; CPU statement e_natten/pytorch.py:46-156).
+ * Same conventions as the 2D calls; the stride arrays are int64_t[3] for the
+ * (batch, head, position) axes, NULL for contiguous; lse is [B, heads, T].
+ */
+int enatten1d_fwd(const void *q, const void *k, const void *v, void *o, float *lse,
+                  int B, int heads, int T, int D, int kernel_size, int dtype,
+                  const int64_t *q_strides, const int64_t *k_strides,
+                  const int64_t *v_strides, float scale, void *stream);
+size_t enatten1d_bwd_workspace_bytes(int B, int heads, int T);
+int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o,
+                  const void *d_o, const float *lse, void *dq, void *dk, void *dv,
+                  void *workspace, int B, int heads, int T, int D, int kernel_size,
+                  int dtype, const int64_t *q_strides, const int64_t *k_strides,
+                  const int64_t *v_strides, float scale, void *stream);
+
+/*
  * Per-kernel timing aid for benchmarks (no counterpart in the reference, whose
  * bench.py:28,59 times whole calls with triton.testing.do_bench).  While
  * enabled, every kernel this library launches is bracketed by HIP events on the

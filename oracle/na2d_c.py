@@ -35,6 +35,10 @@ def lib() -> ctypes.CDLL:
         L.na2d_fwd_f32.argtypes = [fp] * 5 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int]
         L.na2d_bwd_f32.restype = None
         L.na2d_bwd_f32.argtypes = [fp] * 7 + [ctypes.c_int] * 5 + [ctypes.c_float, ctypes.c_int]
+        L.na2d_fwd_rect_f32.restype = None
+        L.na2d_fwd_rect_f32.argtypes = [fp] * 5 + [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_int]
+        L.na2d_bwd_rect_f32.restype = None
+        L.na2d_bwd_rect_f32.argtypes = [fp] * 7 + [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_int]
         _lib = L
     return _lib
 
@@ -75,4 +79,24 @@ def backward(q, k, v, d_o, kernel_size: int, scale: float = 1.0, nthreads: int =
     dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
     lib().na2d_bwd_f32(_p(q), _p(k), _p(v), _p(d_o), _p(dq), _p(dk), _p(dv),
                        B * N, H, W, D, kernel_size, scale, nthreads)
+    return dq, dk, dv
+
+
+def forward_1d(q, k, v, kernel_size: int, scale: float = 1.0, nthreads: int = 0):
+    """1D operator on [B, heads, T, d]: (O, LSE) through the 1 x k rectangular window."""
+    q, k, v = _prep(q, k, v)
+    B, N, T, D = q.shape
+    o = torch.empty_like(q)
+    lse = torch.empty(B, N, T, dtype=torch.float32)
+    lib().na2d_fwd_rect_f32(_p(q), _p(k), _p(v), _p(o), _p(lse), B * N, 1, T, D, 1,
+                            kernel_size, scale, nthreads)
+    return o, lse
+
+
+def backward_1d(q, k, v, d_o, kernel_size: int, scale: float = 1.0, nthreads: int = 0):
+    q, k, v, d_o = _prep(q, k, v, d_o)
+    B, N, T, D = q.shape
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    lib().na2d_bwd_rect_f32(_p(q), _p(k), _p(v), _p(d_o), _p(dq), _p(dk), _p(dv),
+                            B * N, 1, T, D, 1, kernel_size, scale, nthreads)
     return dq, dk, dv

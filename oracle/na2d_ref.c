@@ -57,45 +57,47 @@ int na2d_max_threads(void) {
 
 /* softmax probabilities of one query over its k*k window; returns log-sum-exp */
 static double window_softmax(const float *qv, const float *kslab, int W, int D,
-                             int x0, int y0, int ks, double scale, double *p) {
+                             int x0, int y0, int kh, int kw, double scale, double *p) {
     double m = -INFINITY;
-    for (int a = 0; a < ks; a++)
-        for (int c = 0; c < ks; c++) {
+    for (int a = 0; a < kh; a++)
+        for (int c = 0; c < kw; c++) {
             const float *kv = kslab + ((size_t)(x0 + a) * W + (y0 + c)) * D;
             double s = 0.0;
             for (int e = 0; e < D; e++) s += (double)qv[e] * (double)kv[e];
             s *= scale;
-            p[a * ks + c] = s;
+            p[a * kw + c] = s;
             if (s > m) m = s;
         }
     double z = 0.0;
-    for (int j = 0; j < ks * ks; j++) { p[j] = exp(p[j] - m); z += p[j]; }
-    for (int j = 0; j < ks * ks; j++) p[j] /= z;
+    for (int j = 0; j < kh * kw; j++) { p[j] = exp(p[j] - m); z += p[j]; }
+    for (int j = 0; j < kh * kw; j++) p[j] /= z;
     return m + log(z);
 }
 
-void na2d_fwd_f32(const float *q, const float *k, const float *v, float *o,
-                  float *lse, int S, int H, int W, int D, int ks, float scale,
-                  int nthreads) {
+/* Rectangular kh x kw window; kh = 1 with H = 1 is the 1D operator of
+ * pytorch.py:46-156 (same window rule along the one axis). */
+void na2d_fwd_rect_f32(const float *q, const float *k, const float *v, float *o,
+                       float *lse, int S, int H, int W, int D, int kh, int kw,
+                       float scale, int nthreads) {
     set_threads(nthreads);
     const size_t slab = (size_t)H * W * D;
 #pragma omp parallel
     {
-        double *p = (double *)malloc(sizeof(double) * ks * ks);
+        double *p = (double *)malloc(sizeof(double) * kh * kw);
         double *acc = (double *)malloc(sizeof(double) * D);
 #pragma omp for collapse(2) schedule(static)
         for (int s = 0; s < S; s++)
             for (int x = 0; x < H; x++) {
-                int x0 = na2d_win_start(x, H, ks);
+                int x0 = na2d_win_start(x, H, kh);
                 for (int y = 0; y < W; y++) {
-                    int y0 = na2d_win_start(y, W, ks);
+                    int y0 = na2d_win_start(y, W, kw);
                     size_t qi = s * slab + ((size_t)x * W + y) * D;
-                    double l = window_softmax(q + qi, k + s * slab, W, D, x0, y0, ks, scale, p);
+                    double l = window_softmax(q + qi, k + s * slab, W, D, x0, y0, kh, kw, scale, p);
                     for (int e = 0; e < D; e++) acc[e] = 0.0;
-                    for (int a = 0; a < ks; a++)
-                        for (int c = 0; c < ks; c++) {
+                    for (int a = 0; a < kh; a++)
+                        for (int c = 0; c < kw; c++) {
                             const float *vv = v + s * slab + ((size_t)(x0 + a) * W + (y0 + c)) * D;
-                            double pj = p[a * ks + c];
+                            double pj = p[a * kw + c];
                             for (int e = 0; e < D; e++) acc[e] += pj * (double)vv[e];
                         }
                     for (int e = 0; e < D; e++) o[qi + e] = (float)acc[e];
@@ -107,12 +109,18 @@ void na2d_fwd_f32(const float *q, const float *k, const float *v, float *o,
     }
 }
 
-void na2d_bwd_f32(const float *q, const float *k, const float *v, const float *d_o,
-                  float *dq, float *dk, float *dv, int S, int H, int W, int D,
-                  int ks, float scale, int nthreads) {
+void na2d_fwd_f32(const float *q, const float *k, const float *v, float *o,
+                  float *lse, int S, int H, int W, int D, int ks, float scale,
+                  int nthreads) {
+    na2d_fwd_rect_f32(q, k, v, o, lse, S, H, W, D, ks, ks, scale, nthreads);
+}
+
+void na2d_bwd_rect_f32(const float *q, const float *k, const float *v, const float *d_o,
+                       float *dq, float *dk, float *dv, int S, int H, int W, int D,
+                       int kh, int kw, float scale, int nthreads) {
     set_threads(nthreads);
     const size_t slab = (size_t)H * W * D;
-    const int kk = ks * ks;
+    const int kk = kh * kw;
     /* P and dS of every query, kept so the key-side gather can read them */
     double *P = (double *)malloc(sizeof(double) * (size_t)S * H * W * kk);
     double *dS = (double *)malloc(sizeof(double) * (size_t)S * H * W * kk);
@@ -125,19 +133,19 @@ void na2d_bwd_f32(const float *q, const float *k, const float *v, const float *d
 #pragma omp for collapse(2) schedule(static)
         for (int s = 0; s < S; s++)
             for (int x = 0; x < H; x++) {
-                int x0 = na2d_win_start(x, H, ks);
+                int x0 = na2d_win_start(x, H, kh);
                 for (int y = 0; y < W; y++) {
-                    int y0 = na2d_win_start(y, W, ks);
+                    int y0 = na2d_win_start(y, W, kw);
                     size_t tok = (size_t)s * H * W + (size_t)x * W + y;
                     size_t qi = s * slab + ((size_t)x * W + y) * D;
                     double *p = P + tok * kk, *ds = dS + tok * kk;
-                    window_softmax(q + qi, k + s * slab, W, D, x0, y0, ks, scale, p);
-                    for (int a = 0; a < ks; a++)
-                        for (int c = 0; c < ks; c++) {
+                    window_softmax(q + qi, k + s * slab, W, D, x0, y0, kh, kw, scale, p);
+                    for (int a = 0; a < kh; a++)
+                        for (int c = 0; c < kw; c++) {
                             const float *vv = v + s * slab + ((size_t)(x0 + a) * W + (y0 + c)) * D;
                             double t = 0.0;
                             for (int e = 0; e < D; e++) t += (double)d_o[qi + e] * (double)vv[e];
-                            dp[a * ks + c] = t;
+                            dp[a * kw + c] = t;
                         }
                     /* Jacobian row i: P_i (delta_ij - P_j) */
                     for (int i = 0; i < kk; i++) {
@@ -147,10 +155,10 @@ void na2d_bwd_f32(const float *q, const float *k, const float *v, const float *d
                         ds[i] = t;
                     }
                     for (int e = 0; e < D; e++) acc[e] = 0.0;
-                    for (int a = 0; a < ks; a++)
-                        for (int c = 0; c < ks; c++) {
+                    for (int a = 0; a < kh; a++)
+                        for (int c = 0; c < kw; c++) {
                             const float *kv = k + s * slab + ((size_t)(x0 + a) * W + (y0 + c)) * D;
-                            double t = ds[a * ks + c];
+                            double t = ds[a * kw + c];
                             for (int e = 0; e < D; e++) acc[e] += t * (double)kv[e];
                         }
                     for (int e = 0; e < D; e++) dq[qi + e] = (float)(acc[e] * scale);
@@ -161,16 +169,16 @@ void na2d_bwd_f32(const float *q, const float *k, const float *v, const float *d
         for (int s = 0; s < S; s++)
             for (int x = 0; x < H; x++) {
                 int qx0, qx1;
-                na2d_inv_range(x, H, ks, &qx0, &qx1);
+                na2d_inv_range(x, H, kh, &qx0, &qx1);
                 for (int y = 0; y < W; y++) {
                     int qy0, qy1;
-                    na2d_inv_range(y, W, ks, &qy0, &qy1);
+                    na2d_inv_range(y, W, kw, &qy0, &qy1);
                     for (int e = 0; e < D; e++) { acc[e] = 0.0; acc2[e] = 0.0; }
                     for (int xi = qx0; xi < qx1; xi++) {
-                        int wx = na2d_win_start(xi, H, ks);
+                        int wx = na2d_win_start(xi, H, kh);
                         for (int yi = qy0; yi < qy1; yi++) {
-                            int wy = na2d_win_start(yi, W, ks);
-                            int slot = (x - wx) * ks + (y - wy);
+                            int wy = na2d_win_start(yi, W, kw);
+                            int slot = (x - wx) * kw + (y - wy);
                             size_t tok = (size_t)s * H * W + (size_t)xi * W + yi;
                             size_t qi = s * slab + ((size_t)xi * W + yi) * D;
                             double a = dS[tok * kk + slot], b = P[tok * kk + slot];
@@ -193,4 +201,10 @@ void na2d_bwd_f32(const float *q, const float *k, const float *v, const float *d
     }
     free(P);
     free(dS);
+}
+
+void na2d_bwd_f32(const float *q, const float *k, const float *v, const float *d_o,
+                  float *dq, float *dk, float *dv, int S, int H, int W, int D,
+                  int ks, float scale, int nthreads) {
+    na2d_bwd_rect_f32(q, k, v, d_o, dq, dk, dv, S, H, W, D, ks, ks, scale, nthreads);
 }

@@ -1,0 +1,88 @@
+"""1D operator (natten1d) on the GPU against the CPU oracle, through the C ABI."""
+import pytest
+import torch
+
+from _util import BF16_REL, FP32_MAX_ABS, O, ensure_built
+from oracle import na1d_oracle as O1
+from oracle import na2d_c
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _lib():
+    assert torch.cuda.is_available()
+    return ensure_built()
+
+
+def _run(shape, dtype, ks, seed=0, scale=1.0):
+    from e_natten_amd import Natten1d
+    g = torch.Generator().manual_seed(seed)
+    q, k, v, d_o = (torch.randn(shape, generator=g).to(dtype) for _ in range(4))
+    ref = O1.natten1d_explicit(q, k, v, d_o, ks, scale)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = Natten1d.apply(qg, kg, vg, ks, scale)
+    o.backward(d_o.cuda())
+    got = tuple(t.detach().cpu() for t in (o, qg.grad, kg.grad, vg.grad))
+    for name, x, r in zip(("O", "dQ", "dK", "dV"), got, (ref[0], ref[2], ref[3], ref[4])):
+        err = O.max_abs_err(x, r) if dtype == torch.float32 else O.rel_err(x, r)
+        tol = FP32_MAX_ABS if dtype == torch.float32 else BF16_REL
+        print("   1d", shape, dtype, "k=%d" % ks, name, "err %.3e" % err, flush=True)
+        assert err <= tol, (name, err)
+    return got, ref
+
+
+@pytest.mark.parametrize("ks", [3, 5, 7, 9, 11])
+def test_reference_test_procedure_1d(ks):
+    # test.py:51: fp32 (B=2, heads=3, T=16, d=2), loss sum(o^2), allclose(atol=1e-5)
+    from e_natten_amd import natten1d
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn((2, 3, 16, 2), generator=g) for _ in range(3))
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    o_ref = O1.natten1d_gather(qr, kr, vr, ks)
+    (o_ref ** 2).sum().backward()
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = natten1d(qg, kg, vg, ks)
+    (o ** 2).sum().backward()
+    for x, r in ((o, o_ref), (qg.grad, qr.grad), (kg.grad, kr.grad), (vg.grad, vr.grad)):
+        assert torch.allclose(x.detach().cpu().double(), r.detach(), atol=1e-5, rtol=1e-5)
+
+
+def test_gradcheck_shape_of_reference():
+    # gradcheck.py:6-15 checks (2, 3, 8, 2), k=7 in double; float32 here against the fp64 oracle
+    _run((2, 3, 8, 2), torch.float32, 7, seed=1)
+
+
+@pytest.mark.parametrize("shape,ks,dtype", [
+    ((2, 4, 1024, 64), 7, torch.bfloat16),
+    ((1, 2, 333, 128), 13, torch.bfloat16),
+    ((1, 2, 50, 32), 5, torch.float16),
+    ((2, 2, 257, 48), 9, torch.float32),
+    ((1, 1, 7, 8), 7, torch.float32),      # window == sequence
+    ((1, 3, 19, 5), 3, torch.float32),     # odd head dim
+    ((1, 2, 40, 16), 1, torch.bfloat16),
+])
+def test_shapes_1d(shape, ks, dtype):
+    _run(shape, dtype, ks, seed=2)
+
+
+def test_scale_and_c_oracle_1d():
+    got, ref = _run((2, 2, 100, 64), torch.float32, 5, seed=3, scale=0.125)
+    g = torch.Generator().manual_seed(3)
+    q, k, v, d_o = (torch.randn((2, 2, 100, 64), generator=g) for _ in range(4))
+    oc, _ = na2d_c.forward_1d(q, k, v, 5, 0.125)
+    assert O.max_abs_err(got[0], oc) < FP32_MAX_ABS
+
+
+def test_strided_and_contract_1d():
+    from e_natten_amd import natten1d
+    g = torch.Generator().manual_seed(4)
+    qkv = torch.randn(2, 64, 3, 4, 32, generator=g).to(torch.bfloat16)  # [B, T, 3, heads, d]
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    ref = O1.natten1d_gather(q.double(), k.double(), v.double(), 7)
+    dev = qkv.cuda()
+    o = natten1d(*(dev[:, :, i].permute(0, 2, 1, 3) for i in range(3)), 7)
+    assert o.shape == q.shape and o.dtype == torch.bfloat16
+    assert O.rel_err(o.cpu(), ref) < BF16_REL
+    with pytest.raises(ValueError):
+        natten1d(dev[:, :, 0], dev[:, :, 1], dev[:, :, 2], 4)

@@ -71,6 +71,26 @@ def test_python_surface_mirrors_reference():
     assert "natten2d" in e_natten_amd.__all__
 
 
+def test_1d_surface_and_validation(lib):
+    from e_natten_amd import Natten1d, _lib, natten1d
+    params = list(inspect.signature(Natten1d.forward).parameters.values())
+    assert [p.name for p in params[:5]] == ["ctx", "q", "k", "v", "kernel_size"]
+    assert params[4].default == 7  # e_natten/triton.py:427
+    q = torch.randn(1, 2, 8, 16)
+    for bad in (4, 0, 9):
+        with pytest.raises(ValueError):
+            natten1d(q, q, q, bad)
+    with pytest.raises(ValueError):
+        natten1d(q[0], q[0], q[0], 3)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        natten1d(q, q, q, 3)
+    f = lambda ks, T=8: lib.enatten1d_fwd(1, 1, 1, 1, None, 1, 1, T, 16, ks, 0, None, None,
+                                          None, 1.0, None)
+    assert f(4) == 1 and "odd" in _lib.last_error()
+    assert f(9) == 1 and "smaller" in _lib.last_error()
+    assert lib.enatten1d_bwd_workspace_bytes(2, 3, 10) == 2 * 3 * 10 * 8
+
+
 def test_python_validation_without_gpu():
     from e_natten_amd import natten2d
     q = torch.randn(1, 1, 8, 8, 16)
