@@ -136,10 +136,15 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    lib.enatten_profile_enable(1)
+    # Per-kernel HIP events inside the timed region: every `period`-th launch of
+    # each kernel is bracketed (a record costs ~3 us of queue time; timing all of
+    # them would stretch the step by ~10%).
+    period = max(1, args.steps // 10)
+    lib.enatten_profile_enable(period)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
+    host_s = time.perf_counter() - t0  # time to enqueue all steps
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     lib.enatten_profile_enable(0)
@@ -193,6 +198,8 @@ def main():
         "metric": "natten2d fwd+bwd useful TFLOP/s (B4 H4 d128 k5 bf16)",
         "value": useful / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "host_enqueue_ms_per_step": host_s * 1e3 / args.steps,
+        "kernel_event_sampling": "every %d-th launch" % period,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": "natten2d fwd+bwd B=%d heads=%d H=W=%d head_dim=%d kernel_size=%d"

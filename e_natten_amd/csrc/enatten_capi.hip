@@ -26,10 +26,12 @@ struct ProfRec { hipEvent_t e0, e1; };
 struct ProfSlot {
     std::vector<ProfRec> recs;  // events are created once and reused
     int used = 0;
+    int calls = 0;
     const char *name = "";
 };
 ProfSlot g_prof[ENATTEN_KERNEL_COUNT];
 bool g_prof_on = false;
+int g_prof_period = 1;  // every g_prof_period-th launch of a kernel is timed
 constexpr int kProfMax = 8192;
 }  // namespace
 
@@ -38,6 +40,7 @@ ProfScope::ProfScope(int kernel_slot, const char *kernel_name, hipStream_t strea
     g_prof[slot].name = kernel_name;
     if (!g_prof_on) return;
     ProfSlot &ps = g_prof[slot];
+    if (ps.calls++ % g_prof_period != 0) return;
     if (ps.used >= kProfMax) return;
     if (ps.used == (int)ps.recs.size()) {
         ProfRec r;
@@ -274,10 +277,15 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, co
 }
 
 int enatten_profile_enable(int on) {
-    const int prev = g_prof_on ? 1 : 0;
-    if (on)
-        for (auto &ps : g_prof) ps.used = 0;
-    g_prof_on = on != 0;
+    const int prev = g_prof_on ? g_prof_period : 0;
+    if (on > 0) {
+        for (auto &ps : g_prof) {
+            ps.used = 0;
+            ps.calls = 0;
+        }
+        g_prof_period = on;
+    }
+    g_prof_on = on > 0;
     return prev;
 }
 

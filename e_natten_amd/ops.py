@@ -4,8 +4,8 @@ Mirrors the reference's Python surface (e_natten/triton.py:487-550): a
 ``torch.autograd.Function`` named ``Natten2d`` whose ``apply`` is exported as
 ``natten2d(q, k, v, kernel_size) -> out`` for ``[B, heads, H, W, d]`` tensors.
 The device work is done by hand-written HIP kernels for gfx950 reached through
-the C ABI of libenatten.so; the two entry points are also registered as torch
-custom ops ``enatten::na2d_fwd`` / ``enatten::na2d_bwd``.  There is no CPU or
+the C ABI of libenatten.so; the same host shims are also registered as torch
+custom ops ``enatten::na2d_fwd`` / ``enatten::na2d_bwd`` (and ``na1d_*``).  There is no CPU or
 eager fallback: tensors must live on the GPU and the library must be built.
 """
 from __future__ import annotations
@@ -60,6 +60,15 @@ def _require_gpu(t: torch.Tensor, what: str) -> None:
         raise RuntimeError("%s: tensors must be on the GPU; this build has no CPU path" % what)
 
 
+def _stream_of(t: torch.Tensor) -> int:
+    """Raw HIP stream that torch orders work on for the tensor's device; that
+    device is made current only if it is not already."""
+    idx = t.device.index
+    if idx is not None and idx != torch.cuda.current_device():
+        torch.cuda.set_device(idx)
+    return torch.cuda.current_stream().cuda_stream
+
+
 def _check(rc: int) -> None:
     if rc != 0:
         msg = _lib.last_error()
@@ -74,12 +83,10 @@ def _fwd_impl(q, k, v, kernel_size: int, scale: float):
     B, N, H, W, D = q.shape
     o = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, N, H, W), dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
-        stream = torch.cuda.current_stream().cuda_stream
-        _check(lib.enatten2d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                 lse.data_ptr(), B, N, H, W, D, kernel_size, _DTYPES[q.dtype],
-                                 _lib.strides4(q), _lib.strides4(k), _lib.strides4(v),
-                                 float(scale), stream))
+    _check(lib.enatten2d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                             lse.data_ptr(), B, N, H, W, D, kernel_size, _DTYPES[q.dtype],
+                             _lib.strides4(q), _lib.strides4(k), _lib.strides4(v),
+                             float(scale), _stream_of(q)))
     return o, lse
 
 
@@ -98,13 +105,11 @@ def _bwd_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
     dk, dv = torch.empty_like(dq), torch.empty_like(dq)
     ws = torch.empty(lib.enatten2d_bwd_workspace_bytes(B, N, H, W), dtype=torch.uint8,
                      device=q.device)
-    with torch.cuda.device(q.device):
-        stream = torch.cuda.current_stream().cuda_stream
-        _check(lib.enatten2d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                 d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                                 dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, kernel_size,
-                                 _DTYPES[q.dtype], _lib.strides4(q), _lib.strides4(k),
-                                 _lib.strides4(v), float(scale), stream))
+    _check(lib.enatten2d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                             d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                             dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, kernel_size,
+                             _DTYPES[q.dtype], _lib.strides4(q), _lib.strides4(k),
+                             _lib.strides4(v), float(scale), _stream_of(q)))
     return dq, dk, dv
 
 
@@ -116,12 +121,10 @@ def _fwd1d_impl(q, k, v, kernel_size: int, scale: float):
     B, N, T, D = q.shape
     o = torch.empty((B, N, T, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, N, T), dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
-        stream = torch.cuda.current_stream().cuda_stream
-        _check(lib.enatten1d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                 lse.data_ptr(), B, N, T, D, kernel_size, _DTYPES[q.dtype],
-                                 _lib.strides3(q), _lib.strides3(k), _lib.strides3(v),
-                                 float(scale), stream))
+    _check(lib.enatten1d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                             lse.data_ptr(), B, N, T, D, kernel_size, _DTYPES[q.dtype],
+                             _lib.strides3(q), _lib.strides3(k), _lib.strides3(v),
+                             float(scale), _stream_of(q)))
     return o, lse
 
 
@@ -140,13 +143,11 @@ def _bwd1d_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
     dk, dv = torch.empty_like(dq), torch.empty_like(dq)
     ws = torch.empty(lib.enatten1d_bwd_workspace_bytes(B, N, T), dtype=torch.uint8,
                      device=q.device)
-    with torch.cuda.device(q.device):
-        stream = torch.cuda.current_stream().cuda_stream
-        _check(lib.enatten1d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                 d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                                 dv.data_ptr(), ws.data_ptr(), B, N, T, D, kernel_size,
-                                 _DTYPES[q.dtype], _lib.strides3(q), _lib.strides3(k),
-                                 _lib.strides3(v), float(scale), stream))
+    _check(lib.enatten1d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                             d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                             dv.data_ptr(), ws.data_ptr(), B, N, T, D, kernel_size,
+                             _DTYPES[q.dtype], _lib.strides3(q), _lib.strides3(k),
+                             _lib.strides3(v), float(scale), _stream_of(q)))
     return dq, dk, dv
 
 
@@ -179,8 +180,7 @@ class Natten2d(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, Q, K, V, kernel_size=7, scale=1.0):
-        _validate(Q, K, V, kernel_size)
-        o, lse = torch.ops.enatten.na2d_fwd(Q, K, V, kernel_size, scale)
+        o, lse = _fwd_impl(Q, K, V, kernel_size, scale)
         ctx.save_for_backward(Q, K, V, o, lse)
         ctx.kernel_size = kernel_size
         ctx.scale = scale
@@ -190,8 +190,7 @@ class Natten2d(torch.autograd.Function):
     @torch.autograd.function.once_differentiable
     def backward(ctx, grad_output):
         Q, K, V, o, lse = ctx.saved_tensors
-        dQ, dK, dV = torch.ops.enatten.na2d_bwd(Q, K, V, o, lse, grad_output,
-                                                 ctx.kernel_size, ctx.scale)
+        dQ, dK, dV = _bwd_impl(Q, K, V, o, lse, grad_output, ctx.kernel_size, ctx.scale)
         return dQ, dK, dV, None, None
 
 
@@ -204,8 +203,7 @@ class Natten1d(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, kernel_size=7, scale=1.0):
-        _validate(q, k, v, kernel_size, 4)
-        o, lse = torch.ops.enatten.na1d_fwd(q, k, v, kernel_size, scale)
+        o, lse = _fwd1d_impl(q, k, v, kernel_size, scale)
         ctx.save_for_backward(q, k, v, o, lse)
         ctx.kernel_size = kernel_size
         ctx.scale = scale
@@ -215,8 +213,7 @@ class Natten1d(torch.autograd.Function):
     @torch.autograd.function.once_differentiable
     def backward(ctx, grad_output):
         q, k, v, o, lse = ctx.saved_tensors
-        dQ, dK, dV = torch.ops.enatten.na1d_bwd(q, k, v, o, lse, grad_output,
-                                                 ctx.kernel_size, ctx.scale)
+        dQ, dK, dV = _bwd1d_impl(q, k, v, o, lse, grad_output, ctx.kernel_size, ctx.scale)
         return dQ, dK, dV, None, None
 
 

@@ -122,12 +122,15 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o,
 /*
  * Per-kernel timing aid for benchmarks (no counterpart in the reference, whose
  * bench.py:28,59 times whole calls with triton.testing.do_bench).  While
- * enabled, every kernel this library launches is bracketed by HIP events on the
- * launch stream.  enatten_profile_enable(1) clears the records and starts,
- * enatten_profile_enable(0) stops.  enatten_profile_read waits for the recorded
- * events of one kernel and returns its launch count and summed duration.
- * At most 8192 launches per kernel are recorded between two enables; further
- * launches run untimed.  Not thread-safe; leave it off in production.
+ * enabled, kernels this library launches are bracketed by HIP events on the
+ * launch stream.  enatten_profile_enable(n), n >= 1, clears the records and
+ * times every n-th launch of each kernel (an event record costs a few
+ * microseconds of queue time, so sampling keeps the timed loop undisturbed);
+ * enatten_profile_enable(0) stops; the return value is the previous setting.
+ * enatten_profile_read waits for the recorded events of one kernel and returns
+ * how many launches were timed and their summed duration.  At most 8192 launches
+ * per kernel are recorded between two enables.  Not thread-safe; leave it off in
+ * production.
  */
 enum { ENATTEN_KERNEL_FWD = 0, ENATTEN_KERNEL_BWD_DQ = 1, ENATTEN_KERNEL_BWD_DKDV = 2,
        ENATTEN_KERNEL_BWD_DKDV_FRAME = 3, /* border tiles, when launched separately */
