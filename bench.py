@@ -24,7 +24,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TF = 2500.0   # dense bf16, published
-KERNELS = ("fwd", "bwd_dq", "bwd_dkdv", "bwd_dkdv_frame")
+KERNELS = ("fwd", "bwd_dq", "bwd_dkdv")
 
 
 def algorithmic_bytes(B, N, H, W, D, esize):
@@ -37,17 +37,6 @@ def algorithmic_bytes(B, N, H, W, D, esize):
     M = q * D * esize
     return {"fwd": 4 * M + 4 * q, "bwd_dq": 5 * M + 4 * q, "bwd_dkdv": 6 * M + 4 * q,
             "path": 11 * M + 8 * q}
-
-
-def dkdv_split(H, W, ks):
-    """Fraction of the 8x8 key tiles that the inner dK/dV kernel serves when the
-    matrix-core path splits that pass into an inner and a frame launch."""
-    tr, tc = (H + 7) // 8, (W + 7) // 8
-    i0 = (ks + 7) // 8
-    nr, nc = (H - ks) // 8 - i0, (W - ks) // 8 - i0
-    if nr <= 0 or nc <= 0:
-        return 0.0
-    return nr * nc / float(tr * tc)
 
 
 def cpu_baseline(shape, ks, dtype, useful_flop, budget_rows=8):
@@ -170,11 +159,6 @@ def main():
         avg_ms = tot.value / n.value
         kern[name] = {"kernel": lib.enatten_profile_kernel_name(i).decode(), "launches": n.value,
                       "avg_us": avg_ms * 1e3, "alg_bytes": alg.get(name, 0)}
-    if "bwd_dkdv_frame" in kern:
-        # the dK/dV pass ran as two launches over disjoint key tiles: split its bytes
-        f = dkdv_split(S, S, ks)
-        kern["bwd_dkdv_frame"]["alg_bytes"] = int(alg["bwd_dkdv"] * (1.0 - f))
-        kern["bwd_dkdv"]["alg_bytes"] = int(alg["bwd_dkdv"] * f)
     for k in kern.values():
         k["GBps"] = k["alg_bytes"] / (k["avg_us"] * 1e-6) / 1e9
     names = list(kern)

@@ -119,8 +119,8 @@ struct Geo {
 struct Sched {
     int t, t_end, step;
 };
-__device__ __forceinline__ Sched make_sched(int ntiles) {
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+__device__ __forceinline__ Sched make_sched(int ntiles, int block, int nblocks) {
+    const int xcd = block & 7, slot = block >> 3, slots = nblocks >> 3;
     const int per = (ntiles + 7) >> 3;
     Sched sc;
     sc.t = xcd * per + slot;
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
 
     const Shape &s = a.s;
-    Sched sc = make_sched(ntiles);
+    Sched sc = make_sched(ntiles, blockIdx.x, gridDim.x);
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS>(lds_k);
     zero_row<D, KS>(lds_v);
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
 
     const Shape &s = a.s;
-    Sched sc = make_sched(ntiles);
+    Sched sc = make_sched(ntiles, blockIdx.x, gridDim.x);
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS>(lds_k);
     zero_row<D, KS>(lds_v);
@@ -608,16 +608,12 @@ __device__ __forceinline__ Tile frame_tile(int t, const TileSet &ts, int N) {
 // queries, a wave's queries are the (4+k-1)^2 halo of its 4x4 keys at a fixed
 // place in it, and the mask depends on the lane only.
 template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_inner_mfma(BwdArgs a,
-                                                                              TileSet ts,
-                                                                              int ntiles) {
+__device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, int ntiles,
+                                           int block, int nblocks, short *lds_q, short *lds_g,
+                                           float2 *lds_stat) {
     using G = Geo<D, KS>;
-    __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
-    __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
-    __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
-
     const Shape &s = a.s;
-    Sched sc = make_sched(ntiles);
+    Sched sc = make_sched(ntiles, block, nblocks);
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS>(lds_q);
     zero_row<D, KS>(lds_g);
@@ -763,16 +759,12 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_inner_mfma(
 
 // Frame tiles: the general case, walked block by block (see above).
 template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_frame_mfma(BwdArgs a,
-                                                                              TileSet ts,
-                                                                              int ntiles) {
+__device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, int ntiles,
+                                           int block, int nblocks, short *lds_q, short *lds_g,
+                                           float2 *lds_stat) {
     using G = Geo<D, KS>;
-    __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
-    __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
-    __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
-
     const Shape &s = a.s;
-    Sched sc = make_sched(ntiles);
+    Sched sc = make_sched(ntiles, block, nblocks);
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS>(lds_q);
     zero_row<D, KS>(lds_g);
@@ -957,6 +949,24 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_frame_mfma(
     }
 }
 
+// One launch for the whole dK/dV pass: the first `inner_blocks` workgroups sweep
+// the inner tiles, the rest the frame tiles, so the two kinds of work overlap on
+// every CU and end together.
+template <bool BF, int D, int KS>
+__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArgs a, TileSet ts,
+                                                                        int n_inner, int n_frame,
+                                                                        int inner_blocks) {
+    using G = Geo<D, KS>;
+    __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
+    __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
+    __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
+    if ((int)blockIdx.x < inner_blocks)
+        dkdv_inner<BF, D, KS>(a, ts, n_inner, blockIdx.x, inner_blocks, lds_q, lds_g, lds_stat);
+    else
+        dkdv_frame<BF, D, KS>(a, ts, n_frame, blockIdx.x - inner_blocks,
+                              gridDim.x - inner_blocks, lds_q, lds_g, lds_stat);
+}
+
 // ------------------------------------------------------------------ dispatch
 template <int D, int KS>
 constexpr bool fits() {
@@ -1031,17 +1041,25 @@ int bwd_launch(const BwdArgs &a, hipStream_t st) {
         }
         const int64_t slabs = (int64_t)a.s.B * a.s.N;
         const int64_t n_inner = slabs * ts.ni_r * ts.ni_c, n_frame = nb - n_inner;
-        if (n_inner > 0) {
-            const int grid = persistent_grid(bwd_dkdv_inner_mfma<BF, D, KS>, n_inner);
-            ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_inner_mfma", st);
-            hipLaunchKernelGGL((bwd_dkdv_inner_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a,
-                               ts, (int)n_inner);
-        }
-        if (n_frame > 0) {
-            const int grid = persistent_grid(bwd_dkdv_frame_mfma<BF, D, KS>, n_frame);
-            ProfScope prof(ENATTEN_KERNEL_BWD_DKDV_FRAME, "bwd_dkdv_frame_mfma", st);
-            hipLaunchKernelGGL((bwd_dkdv_frame_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a,
-                               ts, (int)n_frame);
+        {
+            // Share the resident workgroups in proportion to the work.  Measured cost
+            // of a frame tile in inner tiles: about 2 when the inner tiles are bound
+            // by arithmetic (d <= 64), about 1.15 when they are bound by HBM (d = 128).
+            const double cost = D >= 128 ? 1.15 : 2.0;
+            const int grid = persistent_grid(bwd_dkdv_mfma<BF, D, KS>, nb);
+            int inner_blocks = 0;
+            if (n_frame == 0) {
+                inner_blocks = grid;
+            } else if (n_inner > 0) {
+                const double f = (double)n_inner / ((double)n_inner + cost * (double)n_frame);
+                inner_blocks = (int)(f * grid / 8.0 + 0.5) * 8;
+                if (inner_blocks < 8) inner_blocks = 8;
+                if (inner_blocks > grid - 8) inner_blocks = grid - 8;
+                if (inner_blocks > (n_inner + 7) / 8 * 8) inner_blocks = (int)((n_inner + 7) / 8 * 8);
+            }
+            ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
+            hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, ts,
+                               (int)n_inner, (int)n_frame, inner_blocks);
         }
         return check_launch("enatten2d_bwd");
     } else {

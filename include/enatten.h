@@ -133,8 +133,7 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o,
  * production.
  */
 enum { ENATTEN_KERNEL_FWD = 0, ENATTEN_KERNEL_BWD_DQ = 1, ENATTEN_KERNEL_BWD_DKDV = 2,
-       ENATTEN_KERNEL_BWD_DKDV_FRAME = 3, /* border tiles, when launched separately */
-       ENATTEN_KERNEL_COUNT = 4 };
+       ENATTEN_KERNEL_COUNT = 3 };
 int enatten_profile_enable(int on);
 int enatten_profile_read(int kernel, int *launches, double *total_ms);
 /* Name of the device kernel last launched for that slot ("" if none yet). */
