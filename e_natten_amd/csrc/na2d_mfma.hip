@@ -988,13 +988,16 @@ bool layout_ok(const View &v) {
 }
 
 // Persistent grid: as many workgroups as stay resident at once (8 XCDs x 32 CUs x
-// workgroups per CU), never more than there are tiles.
+// workgroups per CU), never more than there are tiles.  The occupancy of a kernel
+// is queried once.
 template <typename K>
 int persistent_grid(K kernel, int64_t ntiles) {
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess ||
-        per_cu < 1)
-        per_cu = 1;
+    static const int per_cu = [kernel]() {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1)
+            n = 1;
+        return n;
+    }();
     const int64_t per_xcd = (ntiles + 7) / 8;
     const int64_t slots = per_xcd < 32 * (int64_t)per_cu ? per_xcd : 32 * (int64_t)per_cu;
     return (int)(8 * slots);

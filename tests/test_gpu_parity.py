@@ -196,3 +196,35 @@ def test_errors_on_gpu(_lib):
         natten2d(q.double(), q.double(), q.double(), 3)
     with pytest.raises(ValueError):
         natten2d(q, q.half(), q, 3)
+
+
+def test_side_stream_and_graph_replay(_lib):
+    # the launchers use the caller's stream and record nothing that a HIP graph
+    # cannot replay: capture forward+backward once, replay it with eager work and
+    # synchronisations in between, and compare every replay with the eager result
+    from e_natten_amd import Natten2d
+    q, k, v, g = make_inputs((2, 2, 40, 48, 64), BF, 21)
+    dev = torch.device("cuda:0")
+    qs, ks_, vs, gs = (t.to(dev) for t in (q, k, v, g))
+    eager = run_gpu(q, k, v, g, 7)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        o, lse = torch.ops.enatten.na2d_fwd(qs, ks_, vs, 7, 1.0)
+        dq, dk, dv = torch.ops.enatten.na2d_bwd(qs, ks_, vs, o, lse, gs, 7, 1.0)
+    side.synchronize()
+    for x, y in zip((o, dq, dk, dv), eager):
+        assert torch.equal(x.cpu(), y)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o2, lse2 = torch.ops.enatten.na2d_fwd(qs, ks_, vs, 7, 1.0)
+        dq2, dk2, dv2 = torch.ops.enatten.na2d_bwd(qs, ks_, vs, o2, lse2, gs, 7, 1.0)
+    for _ in range(3):
+        for t in (o2, dq2, dk2, dv2):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for x, y in zip((o2, dq2, dk2, dv2), eager):
+            assert torch.equal(x.cpu(), y)
+        _ = (qs.float() @ qs.float().transpose(-1, -2)).sum().item()  # unrelated eager work
