@@ -93,6 +93,7 @@ def main():
     ap.add_argument("--kernel-size", type=int, default=5)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the other image sides")
     ap.add_argument("--simt", action="store_true", help="force the vector-ALU kernels")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run a plain 256 MiB device copy (calibrates rocprofv3 "
@@ -192,6 +193,37 @@ def main():
                    "useful_gflop": useful / 1e9},
         "roofline": roofline,
     }
+    if not args.no_sweep:
+        # the other image sides of the reference's benchmark sweep (bench.py:9,34 there),
+        # wall-clock only, a few steps each
+        sweep = []
+        for side in (32, 64, 256):
+            if side == S:
+                continue
+            shp = (B, N, side, side, D)
+            qs, ks_, vs, gs = (torch.randn(shp, generator=g).to(dtype).to(dev) for _ in range(4))
+            for t in (qs, ks_, vs):
+                t.requires_grad_(True)
+
+            def step_s():
+                return torch.autograd.grad(Natten2d.apply(qs, ks_, vs, ks), (qs, ks_, vs), gs)
+
+            for _ in range(5):
+                step_s()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(20):
+                step_s()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3 / 20
+            qn = B * N * side * side
+            fl = 14.0 * ks * ks * D * qn
+            by = 11 * qn * D * qs.element_size() + 8 * qn
+            sweep.append({"side": side, "ms_per_step": ms, "useful_tflops": fl / ms / 1e9,
+                          "path_frac_of_hbm_peak": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                          "mfma_frac_useful": fl / ms / 1e9 / MFMA_BF16_PEAK_TF})
+            del qs, ks_, vs, gs
+        out["sweep"] = sweep
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(shape, ks, dtype, useful)
         out["cpu_baseline"]["gpu_speedup"] = out["cpu_baseline"]["ms"] / ms_step

@@ -97,6 +97,18 @@ __device__ inline A group_sum(A x) {
 template <typename T> struct LogitAcc { using type = float; };
 template <> struct LogitAcc<float> { using type = double; };
 
+// exp(x) for x <= 0 through the hardware 2^y.  With float64 logits the float32
+// rounding of y = x * log2(e) (up to 4e-6 for |y| ~ 60) is put back to first
+// order: 2^(hi + lo) = 2^hi * (1 + lo * ln 2).
+__device__ inline float exp_neg(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+__device__ inline float exp_neg(double x) {
+    const double y = fmax(x * 1.4426950408889634, -200.0);  // also maps -inf to an exact 0
+    const float hi = (float)y;
+    const float lo = (float)(y - (double)hi);
+    const float e = __builtin_amdgcn_exp2f(hi);
+    return fmaf(e, lo * 0.6931471805599453f, e);
+}
+
 constexpr int tile_w(int qpw) {
     int lg = 0;
     while ((1 << lg) < qpw) lg++;
@@ -173,8 +185,8 @@ __global__ __launch_bounds__(256) void fwd_simt(FwdArgs a, int tiles_x, int tile
             }
             const A sc = group_sum<G>(part) * (A)s.scale;
             const A mn = sc > m ? sc : m;
-            const float corr = expf((float)(m - mn));
-            const float pj = expf((float)(sc - mn));
+            const float corr = exp_neg(m - mn);
+            const float pj = exp_neg(sc - mn);
             l = l * corr + pj;
             m = mn;
 #pragma unroll
@@ -256,7 +268,7 @@ __global__ __launch_bounds__(256) void bwd_dq_simt(BwdArgs a, int tiles_x, int t
                     pd = fmaf(gr[c][e], vr[e], pd);
                 }
             }
-            const float p = expf((float)(group_sum<G>(ps) * (A)s.scale - lse));
+            const float p = exp_neg(group_sum<G>(ps) * (A)s.scale - lse);
             const float ds = p * (group_sum<G>(pd) - delta);
             zsum += p;
             esum += ds;
@@ -329,7 +341,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_simt(BwdArgs a, int tiles_x, int
                 }
             }
             const float p =
-                expf((float)(group_sum<G>(ps) * (A)s.scale - (A)a.lse[qtok])) * a.zinv[qtok];
+                exp_neg(group_sum<G>(ps) * (A)s.scale - (A)a.lse[qtok]) * a.zinv[qtok];
             const float ds = p * (group_sum<G>(pd) - a.delta[qtok]);
 #pragma unroll
             for (int c = 0; c < CH; c++)
