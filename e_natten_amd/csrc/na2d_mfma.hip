@@ -92,7 +92,13 @@ struct Geo {
     static constexpr int HR = TH + KS - 1;        // halo of the workgroup tile
     static constexpr int HC = TW + KS - 1;
     static constexpr int SW = 4 + KS - 1;         // halo side of one wave's 4x4 block
-    static constexpr int NK = SW * SW;            // halo tokens per wave
+    // The wave numbers its halo tokens row-major with SWC tokens per row.  SWC is
+    // SW, except that a 14-wide halo (k = 11) is numbered 16 per row: 14 * 16 is a
+    // multiple of 32 like the padded 14 * 14 would be, so no work is added, and the
+    // token -> (row, column) arithmetic becomes shifts (divisions by 14 cost the
+    // k = 11 kernels more registers than they have).
+    static constexpr int SWC = SW == 14 ? 16 : SW;
+    static constexpr int NK = SW * SWC;           // token numbers per wave (some unused)
     static constexpr int NKP = (NK + 31) / 32 * 32;
     static constexpr int MT = NKP / 16;           // 16-token MFMA row tiles
     static constexpr int KSTEPS = NKP / 32;       // reduction steps of the second product
@@ -110,6 +116,12 @@ struct Geo {
     // waves per SIMD to budget registers for: one per workgroup that LDS admits
     // on a CU (a workgroup puts one wave on each of the four SIMDs), at most 2
     static constexpr int WAVES = 2 * LDS_BYTES <= 160 * 1024 ? 2 : 1;
+    // staged LDS row of wave token tk whose halo starts at (orow, ocol) of the
+    // staged block; numbers that are no token read the all-zero row
+    static __device__ __forceinline__ int token_row(int tk, int orow, int ocol) {
+        const int r = tk / SWC, c = tk % SWC;
+        return (tk < NK && c < SW) ? (orow + r) * HC + ocol + c : (int)ZROW;
+    }
 };
 
 // Persistent, XCD-aware tile schedule.  Hardware deals consecutive workgroup ids
@@ -303,9 +315,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
                 const int kk = mt * 16 + n;
-                const int row = kk < G::NK
-                                    ? (lq.orow + kk / G::SW) * G::HC + lq.ocol + kk % G::SW
-                                    : G::ZROW;
+                const int row = G::token_row(kk, lq.orow, lq.ocol);
                 const short *kp = lds_k + row * G::PITCH + g * 8;
                 f32x4 c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -314,7 +324,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int tk = mt * 16 + g * 4 + i;  // halo token of accumulator row g*4+i
-                    const int kr = tk / G::SW, kc = tk % G::SW;
+                    const int kr = tk / G::SWC, kc = tk % G::SWC;
                     const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
                                     (unsigned)(kc - lq.dc) < (unsigned)KS;
                     c[i] = ok ? c[i] * sc2 : -INFINITY;
@@ -346,9 +356,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
                     const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
-                    const int row = tk < G::NK
-                                        ? (lq.orow + tk / G::SW) * G::HC + lq.ocol + tk % G::SW
-                                        : G::ZROW;
+                    const int row = G::token_row(tk, lq.orow, lq.ocol);
                     vp[h] = lds_v + row * G::PITCH + (n & 3) * (D / 4);
                 }
 #pragma unroll
@@ -451,14 +459,19 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
         if (lq.wave_on) {
             // P^T and dP^T on the halo; delta = sum_j P_j dP_j (= dO . O) comes from
             // the same values that form dS, so sum_j dS_j vanishes to rounding
-            f32x4 pr[G::MT], dp[G::MT];
+            // P is kept rounded to 16 bits (it is about to be rounded into dS
+            // anyway) in the registers that will hold dS.  dP stays float32; with
+            // the largest halos it is not kept but formed a second time once delta
+            // is known (measured faster there: the matrix cores are idle, the
+            // registers are not).
+            constexpr bool kKeepDp = !(G::WAVES == 1 && G::MT >= 16);
+            f32x4 dp[kKeepDp ? G::MT : 1];
+            s16x8 dsb[G::KSTEPS];
             float dpart = 0.f;
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
                 const int kk = mt * 16 + n;
-                const int row = kk < G::NK
-                                    ? (lq.orow + kk / G::SW) * G::HC + lq.ocol + kk % G::SW
-                                    : G::ZROW;
+                const int row = G::token_row(kk, lq.orow, lq.ocol);
                 const short *kp = lds_k + row * G::PITCH + g * 8;
                 const short *vp = lds_v + row * G::PITCH + g * 8;
                 f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
@@ -470,22 +483,35 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int tk = mt * 16 + g * 4 + i;
-                    const int kr = tk / G::SW, kc = tk % G::SW;
+                    const int kr = tk / G::SWC, kc = tk % G::SWC;
                     const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
                                     (unsigned)(kc - lq.dc) < (unsigned)KS;
                     cs[i] = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - lse2 : -INFINITY);
                     dpart = fmaf(cs[i], cp[i], dpart);
+                    dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(cs[i]);
                 }
-                pr[mt] = cs;
-                dp[mt] = cp;
+                if constexpr (kKeepDp) dp[mt] = cp;
             }
             const float delta = col_sum(dpart);
-            s16x8 dsb[G::KSTEPS];
 #pragma unroll
-            for (int mt = 0; mt < G::MT; mt++)
+            for (int mt = 0; mt < G::MT; mt++) {
+                f32x4 cp;
+                if constexpr (kKeepDp) {
+                    cp = dp[mt];
+                } else {
+                    const int row = G::token_row(mt * 16 + n, lq.orow, lq.ocol);
+                    const short *vp = lds_v + row * G::PITCH + g * 8;
+                    cp = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(pr[mt][i] * (dp[mt][i] - delta));
+                    for (int ds = 0; ds < G::DS; ds++)
+                        cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(vp + ds * 32), greg[ds], cp);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float p = cvt32<BF>(dsb[mt >> 1][(mt & 1) * 4 + i]);
+                    dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - delta));
+                }
+            }
 
             f32x4 dq[G::DT];
 #pragma unroll
@@ -496,9 +522,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
                     const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
-                    const int row = tk < G::NK
-                                        ? (lq.orow + tk / G::SW) * G::HC + lq.ocol + tk % G::SW
-                                        : G::ZROW;
+                    const int row = G::token_row(tk, lq.orow, lq.ocol);
                     kp[h] = lds_k + row * G::PITCH + (n & 3) * (D / 4);
                 }
 #pragma unroll
@@ -623,7 +647,7 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
     const float sc2 = s.scale * kLog2e;
     const int orow = (wave >> 1) * 4, ocol = (wave & 1) * 4;
     auto row_of = [&](int tk) __attribute__((always_inline)) {
-        return tk < G::NK ? (orow + tk / G::SW) * G::HC + ocol + tk % G::SW : (int)G::ZROW;
+        return G::token_row(tk, orow, ocol);
     };
 
     const HaloPlan<D, KS> plan = make_plan<D, KS>();
@@ -706,8 +730,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
                     const int tk = mt * 16 + g * 4 + i;  // query of accumulator row g*4+i
                     const float2 st = lds_stat[row_of(tk)];
                     const bool ok = tk < G::NK &&
-                                    (unsigned)(tk / G::SW - (n >> 2)) < (unsigned)KS &&
-                                    (unsigned)(tk % G::SW - (n & 3)) < (unsigned)KS;
+                                    (unsigned)(tk / G::SWC - (n >> 2)) < (unsigned)KS &&
+                                    (unsigned)(tk % G::SWC - (n & 3)) < (unsigned)KS;
                     const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
                     pb[m2 * 4 + i] = cvt16<BF>(p);
                     dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
