@@ -14,7 +14,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libenatten.so")
-SOURCES = ["enatten_capi.hip", "na2d_simt.hip", "na2d_mfma.hip"]
+SOURCES = ["enatten_capi.hip", "na2d_simt.hip", "na2d_mfma.hip", "na2d_mfma_fused.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

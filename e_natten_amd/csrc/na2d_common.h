@@ -51,6 +51,14 @@ __host__ __device__ inline int inv_hi(int i, int L, int k) {
     return i >= L - k ? L : i + (k >> 1) + 1;
 }
 
+// The 8x8 tiles of an image split into an inner rectangle, where no key or query
+// is within reach of the border, and the frame around it.
+struct TileSet {
+    int tiles_r, tiles_c;  // 8x8 tiles per image
+    int ir0, ni_r;         // first inner tile row, number of inner tile rows
+    int ic0, ni_c;         // first inner tile column, number of inner tile columns
+};
+
 void set_error(const char *fmt, ...);
 
 // Brackets one kernel launch with HIP events when profiling is enabled.
@@ -69,6 +77,10 @@ int launch_bwd_simt(const BwdArgs &a, int dtype, hipStream_t st);
 // matrix-core kernels: bf16 / f16, D in {32, 64, 128}, square odd window
 bool mfma_supported(int D, int ks, int dtype);
 int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st);
-int launch_bwd_mfma(const BwdArgs &a, int dtype, hipStream_t st);
+int launch_bwd_mfma(const BwdArgs &a, int dtype, bool allow_fused, hipStream_t st);
+// fused backward (dQ, dK, dV from one staging) of the inner tiles, where built
+bool fused_bwd_supported(int D, int ks);
+int launch_bwd_fused_inner(const BwdArgs &a, bool bf16, const TileSet &ts, int64_t n_inner,
+                           hipStream_t st);
 
 }  // namespace enatten

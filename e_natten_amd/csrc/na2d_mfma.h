@@ -1,0 +1,373 @@
+// Device helpers shared by the matrix-core (MFMA) kernels for 2D neighborhood
+// attention on gfx950: operand types, tile geometry, the persistent tile schedule
+// and the global -> register -> LDS staging of a tile's halo.
+#pragma once
+
+#include <math.h>
+
+#include "na2d_common.h"
+
+namespace enatten {
+namespace {
+
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes in flight
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+template <bool BF>
+__device__ __forceinline__ f32x4 mfma16(s16x8 a, s16x8 b, f32x4 c) {
+    if constexpr (BF)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+template <bool BF>
+__device__ __forceinline__ short cvt16(float x) {
+    if constexpr (BF) return __builtin_bit_cast(short, (__bf16)x);
+    else return __builtin_bit_cast(short, (_Float16)x);
+}
+
+template <bool BF>
+__device__ __forceinline__ float cvt32(short x) {
+    if constexpr (BF) return __uint_as_float(((uint32_t)(uint16_t)x) << 16);
+    else return (float)__builtin_bit_cast(_Float16, x);
+}
+
+// 4 tokens x 16 channels out of channel-major LDS, transposed: lane i of each
+// 16-lane group receives, for the channel the caller assigned to it, the values
+// of the 4 tokens addressed by lanes {i/4, 4+i/4, 8+i/4, 12+i/4}.
+__device__ __forceinline__ s16x4 lds_read_tr(const short *p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (s16x4 __attribute__((address_space(3))) *)(p));
+}
+
+__device__ __forceinline__ s16x8 cat(s16x4 lo, s16x4 hi) {
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// max / sum over the four lanes that share a query column (l, l^16, l^32, l^48)
+__device__ __forceinline__ float col_max(float x) {
+    x = fmaxf(x, __shfl_xor(x, 16, 64));
+    return fmaxf(x, __shfl_xor(x, 32, 64));
+}
+__device__ __forceinline__ float col_sum(float x) {
+    x += __shfl_xor(x, 16, 64);
+    return x + __shfl_xor(x, 32, 64);
+}
+
+template <int D, int KS>
+struct Geo {
+    static constexpr int TH = 8, TW = 8;          // pixels per workgroup
+    static constexpr int HR = TH + KS - 1;        // halo of the workgroup tile
+    static constexpr int HC = TW + KS - 1;
+    static constexpr int SW = 4 + KS - 1;         // halo side of one wave's 4x4 block
+    // The wave numbers its halo tokens row-major with SWC tokens per row.  SWC is
+    // SW, except that a 14-wide halo (k = 11) is numbered 16 per row: 14 * 16 is a
+    // multiple of 32 like the padded 14 * 14 would be, so no work is added, and the
+    // token -> (row, column) arithmetic becomes shifts (divisions by 14 cost the
+    // k = 11 kernels more registers than they have).
+    static constexpr int SWC = SW == 14 ? 16 : SW;
+    static constexpr int NK = SW * SWC;           // token numbers per wave (some unused)
+    static constexpr int NKP = (NK + 31) / 32 * 32;
+    static constexpr int MT = NKP / 16;           // 16-token MFMA row tiles
+    static constexpr int KSTEPS = NKP / 32;       // reduction steps of the second product
+    static constexpr int PITCH = D + 8;           // LDS row pitch in elements (16 B pad)
+    static constexpr int ROWS = HR * HC + 1;      // + one all-zero row for padding tokens
+    static constexpr int ZROW = HR * HC;
+    static constexpr int CPR = D / 8;             // 16-byte chunks per row
+    static constexpr int DS = D / 32;             // reduction steps over channels
+    static constexpr int DT = D / 16;             // 16-channel MFMA row tiles of the output
+    static constexpr int NCH = HR * HC * CPR;     // 16-byte chunks per staged halo
+    static constexpr int NL = (NCH + 255) / 256;  // chunks per thread
+    static constexpr int NST = (ROWS + 255) / 256;  // per-query statistics per thread
+    static constexpr size_t LDS_BYTES =
+        (size_t)2 * ROWS * PITCH * sizeof(short) + ROWS * 2 * sizeof(float);
+    // waves per SIMD to budget registers for: one per workgroup that LDS admits
+    // on a CU (a workgroup puts one wave on each of the four SIMDs), at most 2
+    static constexpr int WAVES = 2 * LDS_BYTES <= 160 * 1024 ? 2 : 1;
+    // staged LDS row of wave token tk whose halo starts at (orow, ocol) of the
+    // staged block; numbers that are no token read the all-zero row
+    static __device__ __forceinline__ int token_row(int tk, int orow, int ocol) {
+        const int r = tk / SWC, c = tk % SWC;
+        return (tk < NK && c < SW) ? (orow + r) * HC + ocol + c : (int)ZROW;
+    }
+    // the same when the rows of the staged block are kept in LDS cyclically: image
+    // row y of the block sits in row slot y % HR, and rot = (first image row of the
+    // block) % HR
+    static __device__ __forceinline__ int token_row_rot(int tk, int orow, int ocol, int rot) {
+        const int r = tk / SWC, c = tk % SWC;
+        int x = orow + r + rot;
+        x = x >= HR ? x - HR : x;
+        return (tk < NK && c < SW) ? x * HC + ocol + c : (int)ZROW;
+    }
+};
+
+// Persistent, XCD-aware tile schedule.  Hardware deals consecutive workgroup ids
+// round-robin to the 8 XCDs, each with its own L2: every XCD gets one contiguous
+// run of tiles, and the workgroups resident on it sweep that run side by side, so
+// the halos shared by neighbouring tiles meet in the same L2.
+struct Sched {
+    int t, t_end, step;
+};
+__device__ __forceinline__ Sched make_sched(int ntiles, int block, int nblocks) {
+    const int xcd = block & 7, slot = block >> 3, slots = nblocks >> 3;
+    const int per = (ntiles + 7) >> 3;
+    Sched sc;
+    sc.t = xcd * per + slot;
+    sc.t_end = min(ntiles, (xcd + 1) * per);
+    sc.step = slots;
+    return sc;
+}
+
+// The same split over the XCDs, but every workgroup takes one contiguous run of
+// its XCD's tiles.  With tiles numbered down the columns of an image (tile_of_cm)
+// a workgroup then walks down a column, and consecutive tiles share k-1 of their
+// halo's rows, which stay in LDS.
+__device__ __forceinline__ Sched make_runs(int ntiles, int block, int nblocks) {
+    const int xcd = block & 7, slot = block >> 3, slots = nblocks >> 3;
+    const int per = (ntiles + 7) >> 3;
+    const int lo = xcd * per, hi = min(ntiles, lo + per);
+    const int run = (max(hi - lo, 0) + slots - 1) / slots;
+    Sched sc;
+    sc.t = lo + slot * run;
+    sc.t_end = min(hi, sc.t + run);
+    sc.step = 1;
+    return sc;
+}
+
+struct Tile {
+    int bb, nn, r0, c0;
+};
+__device__ __forceinline__ Tile tile_of_cm(int t, int tiles_r, int tiles_c, int N) {
+    Tile tl;
+    tl.r0 = (t % tiles_r) * 8; t /= tiles_r;
+    tl.c0 = (t % tiles_c) * 8; t /= tiles_c;
+    tl.bb = t / N; tl.nn = t % N;
+    return tl;
+}
+__device__ __forceinline__ Tile tile_of(int t, int tiles_r, int tiles_c, int N) {
+    Tile tl;
+    tl.c0 = (t % tiles_c) * 8; t /= tiles_c;
+    tl.r0 = (t % tiles_r) * 8; t /= tiles_r;
+    tl.bb = t / N; tl.nn = t % N;
+    return tl;
+}
+
+// Staging plan of one thread: which 16-byte chunks of a halo it moves.  Chunk i of
+// thread t is chunk number t + 256*i of the halo in (row, column, channel-chunk)
+// order.  The plan is the same for every tile, so it is computed once.
+template <int D, int KS>
+struct HaloPlan {
+    int rc[Geo<D, KS>::NL];  // halo row << 8 | halo column of chunk i
+    int ch8;                 // first channel of the thread's chunks
+    int lds0;                // LDS element offset of chunk 0
+};
+template <int D, int KS>
+__device__ __forceinline__ HaloPlan<D, KS> make_plan() {
+    using G = Geo<D, KS>;
+    static_assert(256 % G::CPR == 0, "a thread keeps one channel chunk");
+    HaloPlan<D, KS> pl;
+    pl.ch8 = (threadIdx.x % G::CPR) * 8;
+    pl.lds0 = (threadIdx.x / G::CPR) * G::PITCH + pl.ch8;
+#pragma unroll
+    for (int i = 0; i < G::NL; i++) {
+        int row = threadIdx.x / G::CPR + i * (256 / G::CPR);
+        row = row < G::HR * G::HC ? row : G::HR * G::HC - 1;  // tail: harmless duplicate
+        pl.rc[i] = ((row / G::HC) << 8) | (row % G::HC);
+    }
+    return pl;
+}
+template <int D, int KS>
+struct HaloRegs {
+    u32x4 v[Geo<D, KS>::NL];
+};
+// Global -> registers: this thread's share of the halo with origin (hr0, hc0) of
+// one image.  Halo positions at or beyond (rlim, clim) are not needed by any
+// unmasked product; they are clamped to the last valid row / column so the loads
+// stay in bounds and branch-free (the values only ever meet zero probabilities).
+// Addresses are a uniform base plus a 32-bit per-lane byte offset formed with
+// 24-bit multiplies: strides are below 2^22 elements (checked on the host).
+template <int D, int KS>
+__device__ __forceinline__ void halo_fetch(HaloRegs<D, KS> &reg, const HaloPlan<D, KS> &pl,
+                                  const short *img, int64_t sh, int64_t sw, int hr0, int hc0,
+                                  int rlim, int clim) {
+    using G = Geo<D, KS>;
+    const char *base = reinterpret_cast<const char *>(img + hr0 * sh + hc0 * sw);
+    const unsigned sh2 = (unsigned)sh * 2u, sw2 = (unsigned)sw * 2u;
+    const int rmax = rlim - 1 - hr0, cmax = clim - 1 - hc0;
+#pragma unroll
+    for (int i = 0; i < G::NL; i++) {
+        const unsigned r = (unsigned)min(pl.rc[i] >> 8, rmax);
+        const unsigned c = (unsigned)min(pl.rc[i] & 255, cmax);
+        const unsigned off = __umul24(r, sh2) + __umul24(c, sw2) + (unsigned)pl.ch8 * 2u;
+        reg.v[i] = *reinterpret_cast<const u32x4 *>(base + off);
+    }
+}
+// Registers -> LDS, channel-major with padded pitch.
+template <int D, int KS>
+__device__ __forceinline__ void halo_commit(short *lds, const HaloPlan<D, KS> &pl,
+                                   const HaloRegs<D, KS> &reg) {
+    using G = Geo<D, KS>;
+#pragma unroll
+    for (int i = 0; i < G::NL; i++) {
+        const int row = threadIdx.x / G::CPR + i * (256 / G::CPR);
+        if (row < G::HR * G::HC)
+            *reinterpret_cast<u32x4 *>(lds + pl.lds0 + i * (256 / G::CPR) * G::PITCH) = reg.v[i];
+    }
+}
+// Row-range variants for halos whose rows are kept in LDS cyclically (image row y
+// in row slot y % HR): move only the `nrows` image rows from y0 on, all HC columns
+// from hc0 on.  A tile that follows its upper neighbour thus loads only the rows
+// the neighbour's halo did not hold.
+template <int D, int KS>
+__device__ __forceinline__ void halo_fetch_rows(HaloRegs<D, KS> &reg, const HaloPlan<D, KS> &pl,
+                                                const short *img, int64_t sh, int64_t sw, int y0,
+                                                int hc0, int nrows, int rlim, int clim) {
+    using G = Geo<D, KS>;
+    const int yb = min(y0, rlim - 1);
+    const char *base = reinterpret_cast<const char *>(img + yb * sh + hc0 * sw);
+    const unsigned sh2 = (unsigned)sh * 2u, sw2 = (unsigned)sw * 2u;
+    const int rmax = rlim - 1 - yb, cmax = clim - 1 - hc0;
+#pragma unroll
+    for (int i = 0; i < G::NL; i++) {
+        const int r = pl.rc[i] >> 8;
+        if (r < nrows) {
+            const unsigned rr = (unsigned)min(r, rmax);
+            const unsigned c = (unsigned)min(pl.rc[i] & 255, cmax);
+            const unsigned off = __umul24(rr, sh2) + __umul24(c, sw2) + (unsigned)pl.ch8 * 2u;
+            reg.v[i] = *reinterpret_cast<const u32x4 *>(base + off);
+        }
+    }
+}
+template <int D, int KS>
+__device__ __forceinline__ void halo_commit_rows(short *lds, const HaloPlan<D, KS> &pl,
+                                                 const HaloRegs<D, KS> &reg, int y0, int nrows) {
+    using G = Geo<D, KS>;
+    const int rot = y0 % G::HR;
+#pragma unroll
+    for (int i = 0; i < G::NL; i++) {
+        const int pix = threadIdx.x / G::CPR + i * (256 / G::CPR);
+        const int r = pl.rc[i] >> 8;
+        if (pix < G::HR * G::HC && r < nrows) {
+            int slot = rot + r;
+            slot = slot >= G::HR ? slot - G::HR : slot;
+            *reinterpret_cast<u32x4 *>(lds + (slot * G::HC + (pl.rc[i] & 255)) * G::PITCH + pl.ch8) =
+                reg.v[i];
+        }
+    }
+}
+// The spare row stays zero for the whole kernel: padding tokens and tokens
+// outside a wave's halo read it, so they add exact zeros to the second product.
+template <int D, int KS>
+__device__ __forceinline__ void zero_row(short *lds) {
+    using G = Geo<D, KS>;
+    if (threadIdx.x < G::CPR)
+        *reinterpret_cast<uint4 *>(lds + G::ZROW * G::PITCH + threadIdx.x * 8) =
+            make_uint4(0, 0, 0, 0);
+}
+
+// What one lane needs to know about its query (forward, dQ) inside a tile.
+struct LaneQ {
+    bool wave_on, live;
+    int qr, qc;      // query pixel, clamped into the image
+    int orow, ocol;  // origin of the wave's halo inside the staged halo
+    int dr, dc;      // window start of this query relative to the wave's halo
+    int hr0, hc0;    // origin of the staged halo in the image
+    int64_t tok;     // flat token index of the query
+};
+template <int KS>
+__device__ __forceinline__ LaneQ lane_query(const Tile &tl, const Shape &s, int wave, int n) {
+    LaneQ q;
+    const int wr0 = tl.r0 + (wave >> 1) * 4, wc0 = tl.c0 + (wave & 1) * 4;
+    q.wave_on = wr0 < s.H && wc0 < s.W;
+    q.live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
+    q.qr = min(wr0 + (n >> 2), s.H - 1);
+    q.qc = min(wc0 + (n & 3), s.W - 1);
+    q.hr0 = win_start(tl.r0, s.H, KS);
+    q.hc0 = win_start(tl.c0, s.W, KS);
+    const int sr0 = win_start(min(wr0, s.H - 1), s.H, KS);
+    const int sc0 = win_start(min(wc0, s.W - 1), s.W, KS);
+    q.orow = sr0 - q.hr0;
+    q.ocol = sc0 - q.hc0;
+    q.dr = win_start(q.qr, s.H, KS) - sr0;
+    q.dc = win_start(q.qc, s.W, KS) - sc0;
+    q.tok = (((int64_t)tl.bb * s.N + tl.nn) * s.H + q.qr) * s.W + q.qc;
+    return q;
+}
+
+template <typename T>
+__device__ __forceinline__ const short *image(const View &v, const Tile &tl) {
+    return static_cast<const short *>(v.ptr) + tl.bb * v.sb + tl.nn * v.sn;
+}
+
+__device__ __forceinline__ Tile inner_tile(int t, const TileSet &ts, int N) {
+    Tile tl;
+    tl.c0 = (ts.ic0 + t % ts.ni_c) * 8; t /= ts.ni_c;
+    tl.r0 = (ts.ir0 + t % ts.ni_r) * 8; t /= ts.ni_r;
+    tl.bb = t / N; tl.nn = t % N;
+    return tl;
+}
+__device__ __forceinline__ Tile frame_tile(int t, const TileSet &ts, int N) {
+    const int per_img = ts.tiles_r * ts.tiles_c - ts.ni_r * ts.ni_c;
+    const int slab = t / per_img;
+    int e = t % per_img;
+    const int top = ts.ir0 * ts.tiles_c, side = ts.tiles_c - ts.ni_c;
+    int tr, tc;
+    if (e < top) {
+        tr = e / ts.tiles_c; tc = e % ts.tiles_c;
+    } else if (e < top + ts.ni_r * side) {
+        e -= top;
+        tr = ts.ir0 + e / side;
+        tc = e % side;
+        tc = tc < ts.ic0 ? tc : tc + ts.ni_c;
+    } else {
+        e -= top + ts.ni_r * side;
+        tr = ts.ir0 + ts.ni_r + e / ts.tiles_c; tc = e % ts.tiles_c;
+    }
+    Tile tl;
+    tl.r0 = tr * 8; tl.c0 = tc * 8;
+    tl.bb = slab / N; tl.nn = slab % N;
+    return tl;
+}
+
+int check_launch(const char *what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+        return ENATTEN_ELAUNCH;
+    }
+    return ENATTEN_OK;
+}
+
+bool layout_ok(const View &v) {
+    return reinterpret_cast<uintptr_t>(v.ptr) % 16 == 0 && v.sb % 8 == 0 && v.sn % 8 == 0 &&
+           v.sh % 8 == 0 && v.sw % 8 == 0 && v.sh < (1 << 22) && v.sw < (1 << 22);
+}
+
+// Persistent grid: as many workgroups as stay resident at once (8 XCDs x 32 CUs x
+// workgroups per CU), never more than there are tiles.  The occupancy of a kernel
+// is queried once.
+template <typename K>
+int persistent_grid(K kernel, int64_t ntiles) {
+    static const int per_cu = [kernel]() {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1)
+            n = 1;
+        return n;
+    }();
+    const int64_t per_xcd = (ntiles + 7) / 8;
+    const int64_t slots = per_xcd < 32 * (int64_t)per_cu ? per_xcd : 32 * (int64_t)per_cu;
+    return (int)(8 * slots);
+}
+
+}  // namespace
+}  // namespace enatten

@@ -25,248 +25,24 @@
 // Forward follows e_natten/triton.py:242-302 per query (window start, mask,
 // softmax, P.V); the log-sum-exp is kept for the backward.
 
-#include <math.h>
 
-#include "na2d_common.h"
+#include "na2d_mfma.h"
 
 namespace enatten {
 namespace {
 
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes in flight
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
-
-template <bool BF>
-__device__ __forceinline__ f32x4 mfma16(s16x8 a, s16x8 b, f32x4 c) {
-    if constexpr (BF)
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
-                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    else
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
-                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-}
-
-template <bool BF>
-__device__ __forceinline__ short cvt16(float x) {
-    if constexpr (BF) return __builtin_bit_cast(short, (__bf16)x);
-    else return __builtin_bit_cast(short, (_Float16)x);
-}
-
-template <bool BF>
-__device__ __forceinline__ float cvt32(short x) {
-    if constexpr (BF) return __uint_as_float(((uint32_t)(uint16_t)x) << 16);
-    else return (float)__builtin_bit_cast(_Float16, x);
-}
-
-// 4 tokens x 16 channels out of channel-major LDS, transposed: lane i of each
-// 16-lane group receives, for the channel the caller assigned to it, the values
-// of the 4 tokens addressed by lanes {i/4, 4+i/4, 8+i/4, 12+i/4}.
-__device__ __forceinline__ s16x4 lds_read_tr(const short *p) {
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (s16x4 __attribute__((address_space(3))) *)(p));
-}
-
-__device__ __forceinline__ s16x8 cat(s16x4 lo, s16x4 hi) {
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
-// max / sum over the four lanes that share a query column (l, l^16, l^32, l^48)
-__device__ __forceinline__ float col_max(float x) {
-    x = fmaxf(x, __shfl_xor(x, 16, 64));
-    return fmaxf(x, __shfl_xor(x, 32, 64));
-}
-__device__ __forceinline__ float col_sum(float x) {
-    x += __shfl_xor(x, 16, 64);
-    return x + __shfl_xor(x, 32, 64);
-}
-
-template <int D, int KS>
-struct Geo {
-    static constexpr int TH = 8, TW = 8;          // pixels per workgroup
-    static constexpr int HR = TH + KS - 1;        // halo of the workgroup tile
-    static constexpr int HC = TW + KS - 1;
-    static constexpr int SW = 4 + KS - 1;         // halo side of one wave's 4x4 block
-    // The wave numbers its halo tokens row-major with SWC tokens per row.  SWC is
-    // SW, except that a 14-wide halo (k = 11) is numbered 16 per row: 14 * 16 is a
-    // multiple of 32 like the padded 14 * 14 would be, so no work is added, and the
-    // token -> (row, column) arithmetic becomes shifts (divisions by 14 cost the
-    // k = 11 kernels more registers than they have).
-    static constexpr int SWC = SW == 14 ? 16 : SW;
-    static constexpr int NK = SW * SWC;           // token numbers per wave (some unused)
-    static constexpr int NKP = (NK + 31) / 32 * 32;
-    static constexpr int MT = NKP / 16;           // 16-token MFMA row tiles
-    static constexpr int KSTEPS = NKP / 32;       // reduction steps of the second product
-    static constexpr int PITCH = D + 8;           // LDS row pitch in elements (16 B pad)
-    static constexpr int ROWS = HR * HC + 1;      // + one all-zero row for padding tokens
-    static constexpr int ZROW = HR * HC;
-    static constexpr int CPR = D / 8;             // 16-byte chunks per row
-    static constexpr int DS = D / 32;             // reduction steps over channels
-    static constexpr int DT = D / 16;             // 16-channel MFMA row tiles of the output
-    static constexpr int NCH = HR * HC * CPR;     // 16-byte chunks per staged halo
-    static constexpr int NL = (NCH + 255) / 256;  // chunks per thread
-    static constexpr int NST = (ROWS + 255) / 256;  // per-query statistics per thread
-    static constexpr size_t LDS_BYTES =
-        (size_t)2 * ROWS * PITCH * sizeof(short) + ROWS * 2 * sizeof(float);
-    // waves per SIMD to budget registers for: one per workgroup that LDS admits
-    // on a CU (a workgroup puts one wave on each of the four SIMDs), at most 2
-    static constexpr int WAVES = 2 * LDS_BYTES <= 160 * 1024 ? 2 : 1;
-    // staged LDS row of wave token tk whose halo starts at (orow, ocol) of the
-    // staged block; numbers that are no token read the all-zero row
-    static __device__ __forceinline__ int token_row(int tk, int orow, int ocol) {
-        const int r = tk / SWC, c = tk % SWC;
-        return (tk < NK && c < SW) ? (orow + r) * HC + ocol + c : (int)ZROW;
-    }
-};
-
-// Persistent, XCD-aware tile schedule.  Hardware deals consecutive workgroup ids
-// round-robin to the 8 XCDs, each with its own L2: every XCD gets one contiguous
-// run of tiles, and the workgroups resident on it sweep that run side by side, so
-// the halos shared by neighbouring tiles meet in the same L2.
-struct Sched {
-    int t, t_end, step;
-};
-__device__ __forceinline__ Sched make_sched(int ntiles, int block, int nblocks) {
-    const int xcd = block & 7, slot = block >> 3, slots = nblocks >> 3;
-    const int per = (ntiles + 7) >> 3;
-    Sched sc;
-    sc.t = xcd * per + slot;
-    sc.t_end = min(ntiles, (xcd + 1) * per);
-    sc.step = slots;
-    return sc;
-}
-
-struct Tile {
-    int bb, nn, r0, c0;
-};
-__device__ __forceinline__ Tile tile_of(int t, int tiles_r, int tiles_c, int N) {
-    Tile tl;
-    tl.c0 = (t % tiles_c) * 8; t /= tiles_c;
-    tl.r0 = (t % tiles_r) * 8; t /= tiles_r;
-    tl.bb = t / N; tl.nn = t % N;
-    return tl;
-}
-
-// Staging plan of one thread: which 16-byte chunks of a halo it moves.  Chunk i of
-// thread t is chunk number t + 256*i of the halo in (row, column, channel-chunk)
-// order.  The plan is the same for every tile, so it is computed once.
-template <int D, int KS>
-struct HaloPlan {
-    int rc[Geo<D, KS>::NL];  // halo row << 8 | halo column of chunk i
-    int ch8;                 // first channel of the thread's chunks
-    int lds0;                // LDS element offset of chunk 0
-};
-template <int D, int KS>
-__device__ __forceinline__ HaloPlan<D, KS> make_plan() {
-    using G = Geo<D, KS>;
-    static_assert(256 % G::CPR == 0, "a thread keeps one channel chunk");
-    HaloPlan<D, KS> pl;
-    pl.ch8 = (threadIdx.x % G::CPR) * 8;
-    pl.lds0 = (threadIdx.x / G::CPR) * G::PITCH + pl.ch8;
-#pragma unroll
-    for (int i = 0; i < G::NL; i++) {
-        int row = threadIdx.x / G::CPR + i * (256 / G::CPR);
-        row = row < G::HR * G::HC ? row : G::HR * G::HC - 1;  // tail: harmless duplicate
-        pl.rc[i] = ((row / G::HC) << 8) | (row % G::HC);
-    }
-    return pl;
-}
-template <int D, int KS>
-struct HaloRegs {
-    u32x4 v[Geo<D, KS>::NL];
-};
-// Global -> registers: this thread's share of the halo with origin (hr0, hc0) of
-// one image.  Halo positions at or beyond (rlim, clim) are not needed by any
-// unmasked product; they are clamped to the last valid row / column so the loads
-// stay in bounds and branch-free (the values only ever meet zero probabilities).
-// Addresses are a uniform base plus a 32-bit per-lane byte offset formed with
-// 24-bit multiplies: strides are below 2^22 elements (checked on the host).
-template <int D, int KS>
-__device__ __forceinline__ void halo_fetch(HaloRegs<D, KS> &reg, const HaloPlan<D, KS> &pl,
-                                  const short *img, int64_t sh, int64_t sw, int hr0, int hc0,
-                                  int rlim, int clim) {
-    using G = Geo<D, KS>;
-    const char *base = reinterpret_cast<const char *>(img + hr0 * sh + hc0 * sw);
-    const unsigned sh2 = (unsigned)sh * 2u, sw2 = (unsigned)sw * 2u;
-    const int rmax = rlim - 1 - hr0, cmax = clim - 1 - hc0;
-#pragma unroll
-    for (int i = 0; i < G::NL; i++) {
-        const unsigned r = (unsigned)min(pl.rc[i] >> 8, rmax);
-        const unsigned c = (unsigned)min(pl.rc[i] & 255, cmax);
-        const unsigned off = __umul24(r, sh2) + __umul24(c, sw2) + (unsigned)pl.ch8 * 2u;
-        reg.v[i] = *reinterpret_cast<const u32x4 *>(base + off);
-    }
-}
-// Registers -> LDS, channel-major with padded pitch.
-template <int D, int KS>
-__device__ __forceinline__ void halo_commit(short *lds, const HaloPlan<D, KS> &pl,
-                                   const HaloRegs<D, KS> &reg) {
-    using G = Geo<D, KS>;
-#pragma unroll
-    for (int i = 0; i < G::NL; i++) {
-        const int row = threadIdx.x / G::CPR + i * (256 / G::CPR);
-        if (row < G::HR * G::HC)
-            *reinterpret_cast<u32x4 *>(lds + pl.lds0 + i * (256 / G::CPR) * G::PITCH) = reg.v[i];
-    }
-}
-// The spare row stays zero for the whole kernel: padding tokens and tokens
-// outside a wave's halo read it, so they add exact zeros to the second product.
-template <int D, int KS>
-__device__ __forceinline__ void zero_row(short *lds) {
-    using G = Geo<D, KS>;
-    if (threadIdx.x < G::CPR)
-        *reinterpret_cast<uint4 *>(lds + G::ZROW * G::PITCH + threadIdx.x * 8) =
-            make_uint4(0, 0, 0, 0);
-}
-
-// What one lane needs to know about its query (forward, dQ) inside a tile.
-struct LaneQ {
-    bool wave_on, live;
-    int qr, qc;      // query pixel, clamped into the image
-    int orow, ocol;  // origin of the wave's halo inside the staged halo
-    int dr, dc;      // window start of this query relative to the wave's halo
-    int hr0, hc0;    // origin of the staged halo in the image
-    int64_t tok;     // flat token index of the query
-};
-template <int KS>
-__device__ __forceinline__ LaneQ lane_query(const Tile &tl, const Shape &s, int wave, int n) {
-    LaneQ q;
-    const int wr0 = tl.r0 + (wave >> 1) * 4, wc0 = tl.c0 + (wave & 1) * 4;
-    q.wave_on = wr0 < s.H && wc0 < s.W;
-    q.live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
-    q.qr = min(wr0 + (n >> 2), s.H - 1);
-    q.qc = min(wc0 + (n & 3), s.W - 1);
-    q.hr0 = win_start(tl.r0, s.H, KS);
-    q.hc0 = win_start(tl.c0, s.W, KS);
-    const int sr0 = win_start(min(wr0, s.H - 1), s.H, KS);
-    const int sc0 = win_start(min(wc0, s.W - 1), s.W, KS);
-    q.orow = sr0 - q.hr0;
-    q.ocol = sc0 - q.hc0;
-    q.dr = win_start(q.qr, s.H, KS) - sr0;
-    q.dc = win_start(q.qc, s.W, KS) - sc0;
-    q.tok = (((int64_t)tl.bb * s.N + tl.nn) * s.H + q.qr) * s.W + q.qc;
-    return q;
-}
-
-template <typename T>
-__device__ __forceinline__ const short *image(const View &v, const Tile &tl) {
-    return static_cast<const short *>(v.ptr) + tl.bb * v.sb + tl.nn * v.sn;
-}
-
 // ------------------------------------------------------------------ forward
-template <bool BF, int D, int KS>
+// ROLL: walk down the columns of an image and keep the halo rows that consecutive
+// tiles share in LDS (see make_runs); otherwise a strided walk over row-major tiles
+// with the whole halo staged per tile.
+template <bool BF, int D, int KS, bool ROLL>
 __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
 
     const Shape &s = a.s;
-    Sched sc = make_sched(ntiles, blockIdx.x, gridDim.x);
+    Sched sc = ROLL ? make_runs(ntiles, blockIdx.x, gridDim.x) : make_sched(ntiles, blockIdx.x, gridDim.x);
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS>(lds_k);
     zero_row<D, KS>(lds_v);
@@ -278,21 +54,36 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
     const HaloPlan<D, KS> plan = make_plan<D, KS>();
     HaloRegs<D, KS> kst, vst;
     s16x8 qnext[G::DS];
-    auto prefetch = [&](const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
-        halo_fetch<D, KS>(kst, plan, image<short>(a.k, tl), a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W);
-        halo_fetch<D, KS>(vst, plan, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
+    // rows [y0, y0 + nr) of the halo are what LDS does not hold yet
+    auto prefetch = [&](const Tile &tl, const LaneQ &lq, int y0, int nr) __attribute__((always_inline)) {
+        if constexpr (ROLL) {
+            halo_fetch_rows<D, KS>(kst, plan, image<short>(a.k, tl), a.k.sh, a.k.sw, y0, lq.hc0, nr, s.H, s.W);
+            halo_fetch_rows<D, KS>(vst, plan, image<short>(a.v, tl), a.v.sh, a.v.sw, y0, lq.hc0, nr, s.H, s.W);
+        } else {
+            halo_fetch<D, KS>(kst, plan, image<short>(a.k, tl), a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W);
+            halo_fetch<D, KS>(vst, plan, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
+        }
         const short *qp = image<short>(a.q, tl) + lq.qr * a.q.sh + lq.qc * a.q.sw + g * 8;
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++)
             qnext[ds] = *reinterpret_cast<const s16x8 *>(qp + ds * 32);
     };
 
-    Tile cur = tile_of(sc.t, tiles_r, tiles_c, s.N);
+    auto pick = [&](int t) __attribute__((always_inline)) {
+        return ROLL ? tile_of_cm(t, tiles_r, tiles_c, s.N) : tile_of(t, tiles_r, tiles_c, s.N);
+    };
+    Tile cur = pick(sc.t);
     LaneQ lq = lane_query<KS>(cur, s, wave, n);
-    prefetch(cur, lq);
+    int y0 = lq.hr0, nr = G::HR;
+    prefetch(cur, lq, y0, nr);
     for (;;) {
-        halo_commit<D, KS>(lds_k, plan, kst);
-        halo_commit<D, KS>(lds_v, plan, vst);
+        if constexpr (ROLL) {
+            halo_commit_rows<D, KS>(lds_k, plan, kst, y0, nr);
+            halo_commit_rows<D, KS>(lds_v, plan, vst, y0, nr);
+        } else {
+            halo_commit<D, KS>(lds_k, plan, kst);
+            halo_commit<D, KS>(lds_v, plan, vst);
+        }
         s16x8 qreg[G::DS];
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) qreg[ds] = qnext[ds];
@@ -303,10 +94,19 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
         Tile nxt = cur;
         LaneQ lqn = lq;
         if (more) {
-            nxt = tile_of(tn, tiles_r, tiles_c, s.N);
+            nxt = pick(tn);
             lqn = lane_query<KS>(nxt, s, wave, n);
-            prefetch(nxt, lqn);
+            // the tile below in the same image keeps the rows the two halos share
+            const bool below = ROLL && nxt.bb == cur.bb && nxt.nn == cur.nn && nxt.c0 == cur.c0 &&
+                               nxt.r0 > cur.r0 && lqn.hr0 < lq.hr0 + G::HR;
+            y0 = below ? lq.hr0 + G::HR : lqn.hr0;
+            nr = below ? lqn.hr0 - lq.hr0 : G::HR;
+            prefetch(nxt, lqn, y0, nr);
         }
+        const int rot = ROLL ? lq.hr0 % G::HR : 0;
+        auto trow = [&](int tk) __attribute__((always_inline)) {
+            return ROLL ? G::token_row_rot(tk, lq.orow, lq.ocol, rot) : G::token_row(tk, lq.orow, lq.ocol);
+        };
 
         if (lq.wave_on) {
             // logits^T [halo token][query], masked, in units of log2
@@ -315,7 +115,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
                 const int kk = mt * 16 + n;
-                const int row = G::token_row(kk, lq.orow, lq.ocol);
+                const int row = trow(kk);
                 const short *kp = lds_k + row * G::PITCH + g * 8;
                 f32x4 c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -356,7 +156,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
                     const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
-                    const int row = G::token_row(tk, lq.orow, lq.ocol);
+                    const int row = trow(tk);
                     vp[h] = lds_v + row * G::PITCH + (n & 3) * (D / 4);
                 }
 #pragma unroll
@@ -398,29 +198,42 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
 // (equal to dO . O, so the forward output is never read), and dQ^T = K^T dS^T with
 // K read back from LDS transposed.  Also writes delta for the dK/dV pass.
 // Per-query math: e_natten/triton.py:383-398.
-template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs a, int tiles_r, int tiles_c,
-                                                   int ntiles) {
+// FRAME: walk only the tiles of the frame of `ts` (the inner tiles are served by
+// the fused backward).
+template <bool BF, int D, int KS, bool FRAME, bool ROLL>
+__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs a, TileSet ts, int ntiles) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
 
     const Shape &s = a.s;
-    Sched sc = make_sched(ntiles, blockIdx.x, gridDim.x);
+    static_assert(!(FRAME && ROLL), "the frame is not walked by columns");
+    Sched sc = ROLL ? make_runs(ntiles, blockIdx.x, gridDim.x) : make_sched(ntiles, blockIdx.x, gridDim.x);
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS>(lds_k);
     zero_row<D, KS>(lds_v);
 
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
+    auto pick = [&](int t) __attribute__((always_inline)) {
+        if constexpr (FRAME) return frame_tile(t, ts, s.N);
+        else if constexpr (ROLL) return tile_of_cm(t, ts.tiles_r, ts.tiles_c, s.N);
+        else return tile_of(t, ts.tiles_r, ts.tiles_c, s.N);
+    };
 
     const HaloPlan<D, KS> plan = make_plan<D, KS>();
     HaloRegs<D, KS> kst, vst;
     s16x8 qnext[G::DS], gnext[G::DS];
     float lse_next = 0.f;
-    auto prefetch = [&](const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
-        halo_fetch<D, KS>(kst, plan, image<short>(a.k, tl), a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W);
-        halo_fetch<D, KS>(vst, plan, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
+    // rows [y0, y0 + nr) of the halo are what LDS does not hold yet
+    auto prefetch = [&](const Tile &tl, const LaneQ &lq, int y0, int nr) __attribute__((always_inline)) {
+        if constexpr (ROLL) {
+            halo_fetch_rows<D, KS>(kst, plan, image<short>(a.k, tl), a.k.sh, a.k.sw, y0, lq.hc0, nr, s.H, s.W);
+            halo_fetch_rows<D, KS>(vst, plan, image<short>(a.v, tl), a.v.sh, a.v.sw, y0, lq.hc0, nr, s.H, s.W);
+        } else {
+            halo_fetch<D, KS>(kst, plan, image<short>(a.k, tl), a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W);
+            halo_fetch<D, KS>(vst, plan, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
+        }
         const short *qp = image<short>(a.q, tl) + lq.qr * a.q.sh + lq.qc * a.q.sw + g * 8;
         const short *gp = static_cast<const short *>(a.d_o) + lq.tok * D + g * 8;
 #pragma unroll
@@ -431,12 +244,18 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
         lse_next = a.lse[lq.tok];
     };
 
-    Tile cur = tile_of(sc.t, tiles_r, tiles_c, s.N);
+    Tile cur = pick(sc.t);
     LaneQ lq = lane_query<KS>(cur, s, wave, n);
-    prefetch(cur, lq);
+    int y0 = lq.hr0, nr = G::HR;
+    prefetch(cur, lq, y0, nr);
     for (;;) {
-        halo_commit<D, KS>(lds_k, plan, kst);
-        halo_commit<D, KS>(lds_v, plan, vst);
+        if constexpr (ROLL) {
+            halo_commit_rows<D, KS>(lds_k, plan, kst, y0, nr);
+            halo_commit_rows<D, KS>(lds_v, plan, vst, y0, nr);
+        } else {
+            halo_commit<D, KS>(lds_k, plan, kst);
+            halo_commit<D, KS>(lds_v, plan, vst);
+        }
         s16x8 qreg[G::DS], greg[G::DS];
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) {
@@ -451,10 +270,19 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
         Tile nxt = cur;
         LaneQ lqn = lq;
         if (more) {
-            nxt = tile_of(tn, tiles_r, tiles_c, s.N);
+            nxt = pick(tn);
             lqn = lane_query<KS>(nxt, s, wave, n);
-            prefetch(nxt, lqn);
+            // the tile below in the same image keeps the rows the two halos share
+            const bool below = ROLL && nxt.bb == cur.bb && nxt.nn == cur.nn && nxt.c0 == cur.c0 &&
+                               nxt.r0 > cur.r0 && lqn.hr0 < lq.hr0 + G::HR;
+            y0 = below ? lq.hr0 + G::HR : lqn.hr0;
+            nr = below ? lqn.hr0 - lq.hr0 : G::HR;
+            prefetch(nxt, lqn, y0, nr);
         }
+        const int rot = ROLL ? lq.hr0 % G::HR : 0;
+        auto trow = [&](int tk) __attribute__((always_inline)) {
+            return ROLL ? G::token_row_rot(tk, lq.orow, lq.ocol, rot) : G::token_row(tk, lq.orow, lq.ocol);
+        };
 
         if (lq.wave_on) {
             // P^T and dP^T on the halo; delta = sum_j P_j dP_j (= dO . O) comes from
@@ -471,7 +299,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
                 const int kk = mt * 16 + n;
-                const int row = G::token_row(kk, lq.orow, lq.ocol);
+                const int row = trow(kk);
                 const short *kp = lds_k + row * G::PITCH + g * 8;
                 const short *vp = lds_v + row * G::PITCH + g * 8;
                 f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
@@ -499,7 +327,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
                 if constexpr (kKeepDp) {
                     cp = dp[mt];
                 } else {
-                    const int row = G::token_row(mt * 16 + n, lq.orow, lq.ocol);
+                    const int row = trow(mt * 16 + n);
                     const short *vp = lds_v + row * G::PITCH + g * 8;
                     cp = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -522,7 +350,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
                     const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
-                    const int row = G::token_row(tk, lq.orow, lq.ocol);
+                    const int row = trow(tk);
                     kp[h] = lds_k + row * G::PITCH + (n & 3) * (D / 4);
                 }
 #pragma unroll
@@ -589,42 +417,6 @@ __device__ __forceinline__ bool next_block(KeyBlock &b) {
     return true;
 }
 
-// The tiles of an image split into an inner rectangle, where no key or query is
-// within reach of the border, and the frame around it.
-struct TileSet {
-    int tiles_r, tiles_c;  // 8x8 tiles per image
-    int ir0, ni_r;         // first inner tile row, number of inner tile rows
-    int ic0, ni_c;         // first inner tile column, number of inner tile columns
-};
-__device__ __forceinline__ Tile inner_tile(int t, const TileSet &ts, int N) {
-    Tile tl;
-    tl.c0 = (ts.ic0 + t % ts.ni_c) * 8; t /= ts.ni_c;
-    tl.r0 = (ts.ir0 + t % ts.ni_r) * 8; t /= ts.ni_r;
-    tl.bb = t / N; tl.nn = t % N;
-    return tl;
-}
-__device__ __forceinline__ Tile frame_tile(int t, const TileSet &ts, int N) {
-    const int per_img = ts.tiles_r * ts.tiles_c - ts.ni_r * ts.ni_c;
-    const int slab = t / per_img;
-    int e = t % per_img;
-    const int top = ts.ir0 * ts.tiles_c, side = ts.tiles_c - ts.ni_c;
-    int tr, tc;
-    if (e < top) {
-        tr = e / ts.tiles_c; tc = e % ts.tiles_c;
-    } else if (e < top + ts.ni_r * side) {
-        e -= top;
-        tr = ts.ir0 + e / side;
-        tc = e % side;
-        tc = tc < ts.ic0 ? tc : tc + ts.ni_c;
-    } else {
-        e -= top + ts.ni_r * side;
-        tr = ts.ir0 + ts.ni_r + e / ts.tiles_c; tc = e % ts.tiles_c;
-    }
-    Tile tl;
-    tl.r0 = tr * 8; tl.c0 = tc * 8;
-    tl.bb = slab / N; tl.nn = slab % N;
-    return tl;
-}
 
 // Inner tiles.  Every key is attended by exactly the queries within k//2 of it
 // and all windows are centred, so the picture is the forward's with the roles of
@@ -997,34 +789,16 @@ constexpr bool fits() {
     return Geo<D, KS>::LDS_BYTES <= 160 * 1024;
 }
 
-int check_launch(const char *what) {
-    const hipError_t e = hipGetLastError();
-    if (e != hipSuccess) {
-        set_error("%s: launch failed: %s", what, hipGetErrorString(e));
-        return ENATTEN_ELAUNCH;
-    }
-    return ENATTEN_OK;
-}
 
-bool layout_ok(const View &v) {
-    return reinterpret_cast<uintptr_t>(v.ptr) % 16 == 0 && v.sb % 8 == 0 && v.sn % 8 == 0 &&
-           v.sh % 8 == 0 && v.sw % 8 == 0 && v.sh < (1 << 22) && v.sw < (1 << 22);
-}
-
-// Persistent grid: as many workgroups as stay resident at once (8 XCDs x 32 CUs x
-// workgroups per CU), never more than there are tiles.  The occupancy of a kernel
-// is queried once.
-template <typename K>
-int persistent_grid(K kernel, int64_t ntiles) {
-    static const int per_cu = [kernel]() {
-        int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1)
-            n = 1;
-        return n;
-    }();
-    const int64_t per_xcd = (ntiles + 7) / 8;
-    const int64_t slots = per_xcd < 32 * (int64_t)per_cu ? per_xcd : 32 * (int64_t)per_cu;
-    return (int)(8 * slots);
+// Keeping shared halo rows in LDS pays where the kernels are bound by the bytes
+// they pull through the CU's memory pipeline (d = 128) and a workgroup walks at
+// least a few tiles down a column; elsewhere its extra address arithmetic costs
+// more than the loads it saves (measured), so it is only built for d = 128.
+template <int D>
+constexpr bool kRollBuilt = D == 128;
+template <int D>
+bool roll_pays(int64_t ntiles, int grid) {
+    return kRollBuilt<D> && ntiles >= (int64_t)4 * grid;
 }
 
 template <bool BF, int D, int KS>
@@ -1033,11 +807,15 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
         using G = Geo<D, KS>;
         const int tiles_r = (a.s.H + G::TH - 1) / G::TH, tiles_c = (a.s.W + G::TW - 1) / G::TW;
         const int64_t nb = (int64_t)a.s.B * a.s.N * tiles_r * tiles_c;
-        const int grid = persistent_grid(fwd_mfma<BF, D, KS>, nb);
+        const int grid = persistent_grid(fwd_mfma<BF, D, KS, false>, nb);
         {
             ProfScope prof(ENATTEN_KERNEL_FWD, "fwd_mfma", st);
-            hipLaunchKernelGGL((fwd_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
-                               tiles_c, (int)nb);
+            if (roll_pays<D>(nb, grid))
+                hipLaunchKernelGGL((fwd_mfma<BF, D, KS, kRollBuilt<D>>), dim3(grid), dim3(256), 0,
+                                   st, a, tiles_r, tiles_c, (int)nb);
+            else
+                hipLaunchKernelGGL((fwd_mfma<BF, D, KS, false>), dim3(grid), dim3(256), 0, st, a,
+                                   tiles_r, tiles_c, (int)nb);
         }
         return check_launch("enatten2d_fwd");
     } else {
@@ -1047,18 +825,12 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
 }
 
 template <bool BF, int D, int KS>
-int bwd_launch(const BwdArgs &a, hipStream_t st) {
+int bwd_launch(const BwdArgs &a, bool allow_fused, hipStream_t st) {
     if constexpr (fits<D, KS>()) {
         using G = Geo<D, KS>;
         const int tiles_r = (a.s.H + G::TH - 1) / G::TH, tiles_c = (a.s.W + G::TW - 1) / G::TW;
         const int64_t nb = (int64_t)a.s.B * a.s.N * tiles_r * tiles_c;
-        {
-            const int grid = persistent_grid(bwd_dq_mfma<BF, D, KS>, nb);
-            ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
-            hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
-                               tiles_c, (int)nb);
-        }
-        // dK/dV: inner tiles (no key or query within reach of the border) and frame
+        // inner tiles (no key or query within reach of the border) and frame
         TileSet ts;
         ts.tiles_r = tiles_r; ts.tiles_c = tiles_c;
         ts.ir0 = (KS + 7) / 8; ts.ic0 = (KS + 7) / 8;
@@ -1068,6 +840,41 @@ int bwd_launch(const BwdArgs &a, hipStream_t st) {
         }
         const int64_t slabs = (int64_t)a.s.B * a.s.N;
         const int64_t n_inner = slabs * ts.ni_r * ts.ni_c, n_frame = nb - n_inner;
+
+        auto rows_like_o = [&](const View &v) {
+            return v.sh == (int64_t)a.s.W * D && v.sw == D;
+        };
+        if (allow_fused && n_inner > 0 && fused_bwd_supported(D, KS) && rows_like_o(a.q) &&
+            rows_like_o(a.k) && rows_like_o(a.v) && (int64_t)a.s.H * a.s.W * D < (1 << 30)) {
+            // inner tiles: dQ, dK, dV from one staging; frame tiles: the two passes
+            // below restricted to the frame (they read delta of inner queries, which
+            // the fused kernel leaves in the workspace)
+            launch_bwd_fused_inner(a, BF, ts, n_inner, st);
+            if (n_frame > 0) {
+                {
+                    const int grid = persistent_grid(bwd_dq_mfma<BF, D, KS, true, false>, n_frame);
+                    ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
+                    hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS, true, false>), dim3(grid), dim3(256),
+                                       0, st, a, ts, (int)n_frame);
+                }
+                const int grid = persistent_grid(bwd_dkdv_mfma<BF, D, KS>, n_frame);
+                ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
+                hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, ts,
+                                   0, (int)n_frame, 0);
+            }
+            return check_launch("enatten2d_bwd");
+        }
+
+        {
+            const int grid = persistent_grid(bwd_dq_mfma<BF, D, KS, false, false>, nb);
+            ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
+            if (roll_pays<D>(nb, grid))
+                hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS, false, kRollBuilt<D>>), dim3(grid),
+                                   dim3(256), 0, st, a, ts, (int)nb);
+            else
+                hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS, false, false>), dim3(grid), dim3(256), 0,
+                                   st, a, ts, (int)nb);
+        }
         {
             // Share the resident workgroups in proportion to the work.  Measured cost
             // of a frame tile in inner tiles: about 2 when the inner tiles are bound
@@ -1095,21 +902,21 @@ int bwd_launch(const BwdArgs &a, hipStream_t st) {
     }
 }
 
-#define ENATTEN_BY_KS(FN, BF, D, ARGS, ST)                       \
+#define ENATTEN_BY_KS(FN, BF, D, ARGS, ...)                      \
     switch ((ARGS).s.kh) {                                       \
-        case 3: return FN<BF, D, 3>(ARGS, ST);                   \
-        case 5: return FN<BF, D, 5>(ARGS, ST);                   \
-        case 7: return FN<BF, D, 7>(ARGS, ST);                   \
-        case 9: return FN<BF, D, 9>(ARGS, ST);                   \
-        case 11: return FN<BF, D, 11>(ARGS, ST);                 \
-        case 13: return FN<BF, D, 13>(ARGS, ST);                 \
+        case 3: return FN<BF, D, 3>(ARGS, __VA_ARGS__);          \
+        case 5: return FN<BF, D, 5>(ARGS, __VA_ARGS__);          \
+        case 7: return FN<BF, D, 7>(ARGS, __VA_ARGS__);          \
+        case 9: return FN<BF, D, 9>(ARGS, __VA_ARGS__);          \
+        case 11: return FN<BF, D, 11>(ARGS, __VA_ARGS__);        \
+        case 13: return FN<BF, D, 13>(ARGS, __VA_ARGS__);        \
     }
 
-#define ENATTEN_BY_D(FN, BF, ARGS, ST)                           \
-    switch ((ARGS).s.D) {                                        \
-        case 32: ENATTEN_BY_KS(FN, BF, 32, ARGS, ST) break;      \
-        case 64: ENATTEN_BY_KS(FN, BF, 64, ARGS, ST) break;      \
-        case 128: ENATTEN_BY_KS(FN, BF, 128, ARGS, ST) break;    \
+#define ENATTEN_BY_D(FN, BF, ARGS, ...)                                  \
+    switch ((ARGS).s.D) {                                                \
+        case 32: ENATTEN_BY_KS(FN, BF, 32, ARGS, __VA_ARGS__) break;     \
+        case 64: ENATTEN_BY_KS(FN, BF, 64, ARGS, __VA_ARGS__) break;     \
+        case 128: ENATTEN_BY_KS(FN, BF, 128, ARGS, __VA_ARGS__) break;   \
     }
 
 bool fits_rt(int D, int ks) {
@@ -1139,15 +946,15 @@ int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st) {
     return ENATTEN_EUNSUPPORTED;
 }
 
-int launch_bwd_mfma(const BwdArgs &a, int dtype, hipStream_t st) {
+int launch_bwd_mfma(const BwdArgs &a, int dtype, bool allow_fused, hipStream_t st) {
     auto al = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
     if (!layout_ok(a.q) || !layout_ok(a.k) || !layout_ok(a.v) || !al(a.o) || !al(a.d_o) ||
         !al(a.dq) || !al(a.dk) || !al(a.dv))
         return launch_bwd_simt(a, dtype, st);
     if (dtype == ENATTEN_BF16) {
-        ENATTEN_BY_D(bwd_launch, true, a, st)
+        ENATTEN_BY_D(bwd_launch, true, a, allow_fused, st)
     } else {
-        ENATTEN_BY_D(bwd_launch, false, a, st)
+        ENATTEN_BY_D(bwd_launch, false, a, allow_fused, st)
     }
     set_error("no matrix-core kernel for head_dim %d, kernel_size %d", a.s.D, a.s.kh);
     return ENATTEN_EUNSUPPORTED;

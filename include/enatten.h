@@ -37,7 +37,8 @@ enum {
 };
 
 /* which kernel family a call is routed to (enatten2d_kernel_path) */
-enum { ENATTEN_PATH_NONE = 0, ENATTEN_PATH_SIMT = 1, ENATTEN_PATH_MFMA = 2 };
+enum { ENATTEN_PATH_NONE = 0, ENATTEN_PATH_SIMT = 1, ENATTEN_PATH_MFMA = 2,
+       ENATTEN_PATH_MFMA_FUSED = 3 /* enatten_set_path only */ };
 
 int enatten_abi_version(void);
 
@@ -52,9 +53,12 @@ const char *enatten_last_error(void);
 int enatten2d_kernel_path(int D, int kernel_size, int dtype);
 
 /*
- * Restrict dispatch: 0 = automatic (default), ENATTEN_PATH_SIMT = never use the
- * matrix-core kernels.  Process-wide; meant for tests and tuning.  Returns the
- * previous setting.
+ * Steer dispatch: 0 = automatic (default), ENATTEN_PATH_SIMT = never use the
+ * matrix-core kernels, ENATTEN_PATH_MFMA_FUSED = matrix-core kernels with the
+ * fused backward (dQ, dK, dV of the inner tiles from one staging of q, k, v, dO)
+ * where it is built (head_dim 128, kernel_size 5, contiguous rows); it reads the
+ * inputs once but is not faster than the two-pass backward yet, so it is opt-in.
+ * Process-wide; meant for tests and tuning.  Returns the previous setting.
  */
 int enatten_set_path(int path);
 
@@ -133,7 +137,7 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o,
  * production.
  */
 enum { ENATTEN_KERNEL_FWD = 0, ENATTEN_KERNEL_BWD_DQ = 1, ENATTEN_KERNEL_BWD_DKDV = 2,
-       ENATTEN_KERNEL_COUNT = 3 };
+       ENATTEN_KERNEL_BWD_FUSED = 3, ENATTEN_KERNEL_COUNT = 4 };
 int enatten_profile_enable(int on);
 int enatten_profile_read(int kernel, int *launches, double *total_ms);
 /* Name of the device kernel last launched for that slot ("" if none yet). */

@@ -64,6 +64,20 @@ def test_config2_bf16_readme_shape(side, path):
     _case((4, 4, side, side, 128), BF, 5, what="C2 side %d" % side)
 
 
+@pytest.mark.parametrize("shape,dtype", [((4, 4, 32, 32, 128), BF), ((2, 2, 64, 64, 128), BF),
+                                         ((4, 4, 128, 128, 128), BF), ((1, 3, 40, 72, 128), F16),
+                                         ((1, 2, 37, 50, 128), BF)])
+def test_fused_backward_path(shape, dtype, _lib):
+    # the opt-in fused backward (inner tiles: dQ, dK, dV from one staging; border
+    # tiles: the two-pass kernels) against the oracle, square, ragged and fp16
+    from e_natten_amd._lib import PATH_MFMA_FUSED
+    prev = _lib.enatten_set_path(PATH_MFMA_FUSED)
+    try:
+        _case(shape, dtype, 5, what="fused backward %s" % (shape,))
+    finally:
+        _lib.enatten_set_path(prev)
+
+
 def test_config2_bf16_side256():
     _case((4, 4, 256, 256, 128), BF, 5, what="C2 side 256")
 
