@@ -316,6 +316,14 @@ __device__ __forceinline__ Tile inner_tile(int t, const TileSet &ts, int N) {
     tl.bb = t / N; tl.nn = t % N;
     return tl;
 }
+// inner tiles numbered down the columns of the inner rectangle
+__device__ __forceinline__ Tile inner_tile_cm(int t, const TileSet &ts, int N) {
+    Tile tl;
+    tl.r0 = (ts.ir0 + t % ts.ni_r) * 8; t /= ts.ni_r;
+    tl.c0 = (ts.ic0 + t % ts.ni_c) * 8; t /= ts.ni_c;
+    tl.bb = t / N; tl.nn = t % N;
+    return tl;
+}
 __device__ __forceinline__ Tile frame_tile(int t, const TileSet &ts, int N) {
     const int per_img = ts.tiles_r * ts.tiles_c - ts.ni_r * ts.ni_c;
     const int slab = t / per_img;

@@ -423,13 +423,13 @@ __device__ __forceinline__ bool next_block(KeyBlock &b) {
 // queries and keys exchanged: the staged block is the tile's (8+k-1)^2 halo of
 // queries, a wave's queries are the (4+k-1)^2 halo of its 4x4 keys at a fixed
 // place in it, and the mask depends on the lane only.
-template <bool BF, int D, int KS>
+template <bool BF, int D, int KS, bool ROLL>
 __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, int ntiles,
                                            int block, int nblocks, short *lds_q, short *lds_g,
                                            float2 *lds_stat) {
     using G = Geo<D, KS>;
     const Shape &s = a.s;
-    Sched sc = make_sched(ntiles, block, nblocks);
+    Sched sc = ROLL ? make_runs(ntiles, block, nblocks) : make_sched(ntiles, block, nblocks);
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS>(lds_q);
     zero_row<D, KS>(lds_g);
@@ -438,24 +438,63 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
     const int orow = (wave >> 1) * 4, ocol = (wave & 1) * 4;
+    int rot = 0;  // ROLL: (first image row of the staged block) % HR
     auto row_of = [&](int tk) __attribute__((always_inline)) {
-        return G::token_row(tk, orow, ocol);
+        return ROLL ? G::token_row_rot(tk, orow, ocol, rot) : G::token_row(tk, orow, ocol);
+    };
+    auto pick = [&](int t) __attribute__((always_inline)) {
+        return ROLL ? inner_tile_cm(t, ts, s.N) : inner_tile(t, ts, s.N);
     };
 
     const HaloPlan<D, KS> plan = make_plan<D, KS>();
     HaloRegs<D, KS> qst, gst;
     float2 sst[G::NST];
-    auto prefetch = [&](const Tile &tl) __attribute__((always_inline)) {
+    // ROLL: rows [y0, y0 + nr) of the block are what LDS does not hold yet
+    auto prefetch = [&](const Tile &tl, int y0, int nr) __attribute__((always_inline)) {
         const int64_t img_tok = ((int64_t)tl.bb * s.N + tl.nn) * s.H * (int64_t)s.W;
         const int br = tl.r0 - KS / 2, bc = tl.c0 - KS / 2;
-        halo_fetch<D, KS>(qst, plan, image<short>(a.q, tl), a.q.sh, a.q.sw, br, bc, s.H, s.W);
-        halo_fetch<D, KS>(gst, plan, static_cast<const short *>(a.d_o) + img_tok * D,
-                          (int64_t)s.W * D, D, br, bc, s.H, s.W);
+        if constexpr (ROLL) {
+            halo_fetch_rows<D, KS>(qst, plan, image<short>(a.q, tl), a.q.sh, a.q.sw, y0, bc, nr, s.H, s.W);
+            halo_fetch_rows<D, KS>(gst, plan, static_cast<const short *>(a.d_o) + img_tok * D,
+                                   (int64_t)s.W * D, D, y0, bc, nr, s.H, s.W);
+        } else {
+            halo_fetch<D, KS>(qst, plan, image<short>(a.q, tl), a.q.sh, a.q.sw, br, bc, s.H, s.W);
+            halo_fetch<D, KS>(gst, plan, static_cast<const short *>(a.d_o) + img_tok * D,
+                              (int64_t)s.W * D, D, br, bc, s.H, s.W);
+        }
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
             const int id = min((int)threadIdx.x + i * 256, G::ZROW - 1);
-            const int64_t qt = img_tok + (int64_t)(br + id / G::HC) * s.W + bc + id % G::HC;
-            sst[i] = make_float2(a.lse[qt] * kLog2e, a.delta[qt]);
+            const int pr = id / G::HC, pc = id % G::HC;
+            if (!ROLL || pr < nr) {
+                const int64_t qt = img_tok + (int64_t)((ROLL ? y0 : br) + pr) * s.W + bc + pc;
+                sst[i] = make_float2(a.lse[qt] * kLog2e, a.delta[qt]);
+            }
+        }
+    };
+    auto commit = [&](int y0, int nr) __attribute__((always_inline)) {
+        if constexpr (ROLL) {
+            halo_commit_rows<D, KS>(lds_q, plan, qst, y0, nr);
+            halo_commit_rows<D, KS>(lds_g, plan, gst, y0, nr);
+            const int r0m = y0 % G::HR;
+#pragma unroll
+            for (int i = 0; i < G::NST; i++) {
+                const int id = threadIdx.x + i * 256;
+                const int pr = id / G::HC, pc = id % G::HC;
+                if (id < G::ZROW && pr < nr) {
+                    int slot = r0m + pr;
+                    slot = slot >= G::HR ? slot - G::HR : slot;
+                    lds_stat[slot * G::HC + pc] = sst[i];
+                }
+            }
+        } else {
+            halo_commit<D, KS>(lds_q, plan, qst);
+            halo_commit<D, KS>(lds_g, plan, gst);
+#pragma unroll
+            for (int i = 0; i < G::NST; i++) {
+                const int id = threadIdx.x + i * 256;
+                if (id < G::ZROW) lds_stat[id] = sst[i];
+            }
         }
     };
     // B operands of a tile: this lane's key, channels ds*32 + g*8 ..  Loaded when
@@ -473,17 +512,12 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         }
     };
 
-    Tile cur = inner_tile(sc.t, ts, s.N);
-    prefetch(cur);
+    Tile cur = pick(sc.t);
+    int y0 = cur.r0 - KS / 2, nr = G::HR;
+    prefetch(cur, y0, nr);
     load_keys(cur);
     for (;;) {
-        halo_commit<D, KS>(lds_q, plan, qst);
-        halo_commit<D, KS>(lds_g, plan, gst);
-#pragma unroll
-        for (int i = 0; i < G::NST; i++) {
-            const int id = threadIdx.x + i * 256;
-            if (id < G::ZROW) lds_stat[id] = sst[i];
-        }
+        commit(y0, nr);
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) asm volatile("" : "+v"(kreg[ds]), "+v"(vreg[ds]));
         __syncthreads();
@@ -491,9 +525,15 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         const int tn = sc.t + sc.step;
         const bool more = tn < sc.t_end;
         Tile nxt = cur;
+        if (ROLL) rot = (cur.r0 - KS / 2) % G::HR;
         if (more) {
-            nxt = inner_tile(tn, ts, s.N);
-            prefetch(nxt);
+            nxt = pick(tn);
+            // the tile below in the same image keeps the rows the two blocks share
+            const bool below = ROLL && nxt.bb == cur.bb && nxt.nn == cur.nn && nxt.c0 == cur.c0 &&
+                               nxt.r0 > cur.r0 && nxt.r0 - cur.r0 < G::HR;
+            y0 = below ? cur.r0 - KS / 2 + G::HR : nxt.r0 - KS / 2;
+            nr = below ? nxt.r0 - cur.r0 : G::HR;
+            prefetch(nxt, y0, nr);
         }
 
         f32x4 dk[G::DT], dv[G::DT];
@@ -768,7 +808,7 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 // One launch for the whole dK/dV pass: the first `inner_blocks` workgroups sweep
 // the inner tiles, the rest the frame tiles, so the two kinds of work overlap on
 // every CU and end together.
-template <bool BF, int D, int KS>
+template <bool BF, int D, int KS, bool ROLL>
 __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArgs a, TileSet ts,
                                                                         int n_inner, int n_frame,
                                                                         int inner_blocks) {
@@ -777,7 +817,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArg
     __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
     __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
     if ((int)blockIdx.x < inner_blocks)
-        dkdv_inner<BF, D, KS>(a, ts, n_inner, blockIdx.x, inner_blocks, lds_q, lds_g, lds_stat);
+        dkdv_inner<BF, D, KS, ROLL>(a, ts, n_inner, blockIdx.x, inner_blocks, lds_q, lds_g, lds_stat);
     else
         dkdv_frame<BF, D, KS>(a, ts, n_frame, blockIdx.x - inner_blocks,
                               gridDim.x - inner_blocks, lds_q, lds_g, lds_stat);
@@ -857,10 +897,10 @@ int bwd_launch(const BwdArgs &a, bool allow_fused, hipStream_t st) {
                     hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS, true, false>), dim3(grid), dim3(256),
                                        0, st, a, ts, (int)n_frame);
                 }
-                const int grid = persistent_grid(bwd_dkdv_mfma<BF, D, KS>, n_frame);
+                const int grid = persistent_grid(bwd_dkdv_mfma<BF, D, KS, false>, n_frame);
                 ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
-                hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, ts,
-                                   0, (int)n_frame, 0);
+                hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, false>), dim3(grid), dim3(256), 0, st,
+                                   a, ts, 0, (int)n_frame, 0);
             }
             return check_launch("enatten2d_bwd");
         }
@@ -880,7 +920,7 @@ int bwd_launch(const BwdArgs &a, bool allow_fused, hipStream_t st) {
             // of a frame tile in inner tiles: about 2 when the inner tiles are bound
             // by arithmetic (d <= 64), about 1.15 when they are bound by HBM (d = 128).
             const double cost = D >= 128 ? 1.15 : 2.0;
-            const int grid = persistent_grid(bwd_dkdv_mfma<BF, D, KS>, nb);
+            const int grid = persistent_grid(bwd_dkdv_mfma<BF, D, KS, false>, nb);
             int inner_blocks = 0;
             if (n_frame == 0) {
                 inner_blocks = grid;
@@ -892,8 +932,12 @@ int bwd_launch(const BwdArgs &a, bool allow_fused, hipStream_t st) {
                 if (inner_blocks > (n_inner + 7) / 8 * 8) inner_blocks = (int)((n_inner + 7) / 8 * 8);
             }
             ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
-            hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, ts,
-                               (int)n_inner, (int)n_frame, inner_blocks);
+            if (inner_blocks > 0 && roll_pays<D>(n_inner, inner_blocks))
+                hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, kRollBuilt<D>>), dim3(grid), dim3(256),
+                                   0, st, a, ts, (int)n_inner, (int)n_frame, inner_blocks);
+            else
+                hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, false>), dim3(grid), dim3(256), 0, st,
+                                   a, ts, (int)n_inner, (int)n_frame, inner_blocks);
         }
         return check_launch("enatten2d_bwd");
     } else {
