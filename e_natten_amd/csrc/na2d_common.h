@@ -78,9 +78,9 @@ int launch_bwd_simt(const BwdArgs &a, int dtype, hipStream_t st);
 bool mfma_supported(int D, int ks, int dtype);
 int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st);
 int launch_bwd_mfma(const BwdArgs &a, int dtype, bool allow_fused, hipStream_t st);
-// fused backward (dQ, dK, dV from one staging) of the inner tiles, where built
-bool fused_bwd_supported(int D, int ks);
-int launch_bwd_fused_inner(const BwdArgs &a, bool bf16, const TileSet &ts, int64_t n_inner,
-                           hipStream_t st);
+// fused backward (dQ, dK, dV of every tile from one staging), where built
+bool fused_bwd_supported(const BwdArgs &a);
+int launch_bwd_fused(const BwdArgs &a, bool bf16, const TileSet &ts, int64_t ntiles,
+                     hipStream_t st);
 
 }  // namespace enatten

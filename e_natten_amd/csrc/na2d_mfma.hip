@@ -881,27 +881,8 @@ int bwd_launch(const BwdArgs &a, bool allow_fused, hipStream_t st) {
         const int64_t slabs = (int64_t)a.s.B * a.s.N;
         const int64_t n_inner = slabs * ts.ni_r * ts.ni_c, n_frame = nb - n_inner;
 
-        auto rows_like_o = [&](const View &v) {
-            return v.sh == (int64_t)a.s.W * D && v.sw == D;
-        };
-        if (allow_fused && n_inner > 0 && fused_bwd_supported(D, KS) && rows_like_o(a.q) &&
-            rows_like_o(a.k) && rows_like_o(a.v) && (int64_t)a.s.H * a.s.W * D < (1 << 30)) {
-            // inner tiles: dQ, dK, dV from one staging; frame tiles: the two passes
-            // below restricted to the frame (they read delta of inner queries, which
-            // the fused kernel leaves in the workspace)
-            launch_bwd_fused_inner(a, BF, ts, n_inner, st);
-            if (n_frame > 0) {
-                {
-                    const int grid = persistent_grid(bwd_dq_mfma<BF, D, KS, true, false>, n_frame);
-                    ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
-                    hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS, true, false>), dim3(grid), dim3(256),
-                                       0, st, a, ts, (int)n_frame);
-                }
-                const int grid = persistent_grid(bwd_dkdv_mfma<BF, D, KS, false>, n_frame);
-                ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
-                hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, false>), dim3(grid), dim3(256), 0, st,
-                                   a, ts, 0, (int)n_frame, 0);
-            }
+        if (allow_fused && fused_bwd_supported(a)) {
+            launch_bwd_fused(a, BF, ts, nb, st);
             return check_launch("enatten2d_bwd");
         }
 

@@ -1,21 +1,29 @@
 // Fused backward of 2D neighborhood attention on the matrix cores of gfx950:
 // dQ, dK and dV of an 8x8 tile of pixels from ONE staging of the tile's
-// (8+k-1)^2 halo of q, k, v and dO, so that the backward reads each input once
-// (the split passes of na2d_mfma.hip read them twice).
+// (8+k-1)^2 block of q, k, v and dO, so that the backward reads each input once
+// (the two passes of na2d_mfma.hip read them twice).
 //
-// A workgroup is eight waves around one copy of the halo in LDS (all four
+// A workgroup is eight waves around one copy of the block in LDS (all four
 // tensors, which is why only one workgroup fits a CU):
-//   waves 0-3  query side: dQ of their 4x4 queries over the keys of the halo
+//   waves 0-3  query side: dQ of their 4x4 queries over the keys of the block
 //              (e_natten/triton.py:383-398 per query);
-//   waves 4-7  key side: dK, dV of their 4x4 keys over the queries of the halo
+//   waves 4-7  key side: dK, dV of their 4x4 keys over the queries of the block
 //              (the inverse neighbourhood of e_natten/pytorch.py:13-23, :261-288).
-// Both sides recompute P from the saved log-sum-exp.  delta = dO . O of the halo's
-// queries is formed while the halo is written to LDS (the forward output is read
+// Both sides recompute P from the saved log-sum-exp.  delta = dO . O of the block's
+// queries is formed while the block is written to LDS (the forward output is read
 // for this and for nothing else).  The MFMA operand layouts, the token numbering
 // and the transposing LDS reads are those of na2d_mfma.hip.
 //
-// The kernel is persistent like the others: the next tile's halo travels from
-// HBM into registers while the current tile is computed out of LDS.
+// The block of the tile at (r0, c0) is the pixels [r0 - k/2, r0 + 8 + k/2) x
+// [c0 - k/2, c0 + 8 + k/2); with image sides that are multiples of 8 it holds
+// every key a query of the tile attends to and every query that attends to a key
+// of the tile, also beside the border (positions outside the image are staged as
+// copies of the nearest pixel and masked).  Workgroups walk down the columns of an
+// image, and the k-1 block rows that consecutive tiles share stay in LDS (image
+// row y in row slot (y + k/2) % HR): a step stages 8 new rows.
+//
+// The kernel is persistent like the others: the next tile's rows travel from HBM
+// into registers while the current tile is computed out of LDS.
 
 #include <type_traits>
 
@@ -27,12 +35,19 @@ namespace {
 template <int D, int KS>
 struct FGeo {
     using G = Geo<D, KS>;
-    static constexpr int NT = 512;                       // threads per workgroup
-    static constexpr int RP = NT / G::CPR;               // halo rows staged per pass
-    static constexpr int NL = (G::HR * G::HC + RP - 1) / RP;  // passes (chunks per thread and tensor)
+    static constexpr int NT = 512;                        // threads per workgroup
+    static constexpr int RP = NT / G::CPR;                // block pixels staged per pass
+    static constexpr int BR = 8;                          // block rows staged per step
+    static constexpr int NL = (BR * G::HC + RP - 1) / RP; // passes per step
+    // Key side beside the border: the queries that attend to a wave's 4x4 keys
+    // span up to SW + k/2 rows and columns there; they are numbered 16 per row.
+    static constexpr int SWB = G::SW + KS / 2;
+    static constexpr int MTB = (SWB + 1) / 2 * 2;         // one MFMA row tile per row, even
+    static constexpr int KSB = MTB / 2;
     static constexpr size_t LDS_BYTES =
-        (size_t)4 * G::ROWS * G::PITCH * sizeof(short) + (size_t)2 * G::ROWS * sizeof(float);
-    static constexpr bool FITS = LDS_BYTES <= 160 * 1024;
+        (size_t)4 * G::ROWS * G::PITCH * sizeof(short) + (size_t)G::ROWS * sizeof(float2);
+    static constexpr bool FITS = LDS_BYTES <= 160 * 1024 && G::HR - BR <= BR && SWB <= 16 &&
+                                 SWB <= G::HR;
 };
 
 template <int NL>
@@ -77,6 +92,7 @@ template <bool BF, int D, int KS>
 __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int ntiles) {
     using G = Geo<D, KS>;
     using F = FGeo<D, KS>;
+    constexpr int HALF = KS / 2;
     __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
@@ -84,7 +100,45 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     __shared__ float2 lds_stat[G::ROWS];  // (log-sum-exp * log2(e), dO . O) per staged query
 
     const Shape &s = a.s;
-    Sched sc = make_sched(ntiles, blockIdx.x, gridDim.x);
+    // Contiguous runs of column-major tiles per workgroup like make_runs, but of equal
+    // cost rather than equal length: a tile beside the border costs about 1.5 inner
+    // tiles here (measured), and whole columns of them (the first and last column of
+    // every image) would otherwise make their workgroups the last to finish.
+    Sched sc;
+    {
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+        const int per = (ntiles + 7) >> 3;
+        const int lo = xcd * per, hi = min(ntiles, lo + per);
+        const int per_img = ts.tiles_r * ts.tiles_c;
+        // cost of tiles [0, t) in column-major order: 2 per inner tile, 3 per border tile
+        auto cost_to = [&](int t) __attribute__((always_inline)) {
+            const int img = t / per_img, e = t % per_img;
+            const int col = e / ts.tiles_r, row = e % ts.tiles_r;
+            auto inner_in_col = [&](int c, int rows) __attribute__((always_inline)) {
+                const bool cin = c >= ts.ic0 && c < ts.ic0 + ts.ni_c;
+                return cin ? max(0, min(rows, ts.ir0 + ts.ni_r) - ts.ir0) : 0;
+            };
+            const int full_inner_cols = max(0, min(col, ts.ic0 + ts.ni_c) - ts.ic0);
+            const long long inner = (long long)img * ts.ni_r * ts.ni_c +
+                                    (long long)full_inner_cols * ts.ni_r + inner_in_col(col, row);
+            return 3ll * t - inner;
+        };
+        const long long c_lo = cost_to(lo), c_hi = cost_to(max(hi, lo));
+        auto start_of = [&](int k) __attribute__((always_inline)) {
+            // first tile t in [lo, hi] with cost_to(t) - c_lo >= k * (c_hi - c_lo) / slots
+            const long long want = c_lo + (c_hi - c_lo) * k / slots;
+            int a0 = lo, a1 = max(hi, lo);
+            while (a0 < a1) {
+                const int mid = (a0 + a1) >> 1;
+                if (cost_to(mid) >= want) a1 = mid;
+                else a0 = mid + 1;
+            }
+            return a0;
+        };
+        sc.t = start_of(slot);
+        sc.t_end = slot + 1 == slots ? max(hi, lo) : start_of(slot + 1);
+        sc.step = 1;
+    }
     if (sc.t >= sc.t_end) return;
     const int tid = threadIdx.x;
     if (tid < G::CPR) {
@@ -96,96 +150,169 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     }
     if (tid == 0) lds_stat[G::ZROW] = make_float2(0.f, 0.f);
 
-    const int wave = tid >> 6, l = tid & 63, n = l & 15, g = l >> 4;
+    // the wave number through readfirstlane, so that the compiler knows it is uniform:
+    // the role branch is then a scalar branch and per-wave values live in SGPRs
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63;
     const int role = wave >> 2, w = wave & 3;
     const float sc2 = s.scale * kLog2e;
-    // origin of the wave's (4+k-1)^2 halo inside the staged block, and the place of
-    // this lane's pixel (query or key) in the block
-    const int orow = (w >> 1) * 4, ocol = (w & 1) * 4;
-    const int prow = (KS / 2 + orow + (n >> 2)) * G::HC + KS / 2 + ocol + (n & 3);
-    auto row_of = [&](int tk) __attribute__((always_inline)) {
-        return G::token_row(tk, orow, ocol);
-    };
 
-    // staging plan: chunk i of this thread is channel chunk tid % CPR of block row
-    // tid / CPR + i * RP
-    const int ch8 = (tid % G::CPR) * 8;
-    const int srow = tid / G::CPR;
+    // ---- staging: a step moves BR rows x HC columns of the block, all five tensors.
+    // Chunk i of this thread is channel chunk tid % CPR of pixel tid / CPR + i * RP of
+    // the step (row-major).  q, k, v rows are laid out like dO and O here (stride W*D
+    // between rows, D between pixels; checked on the host), so one set of offsets
+    // serves all five tensors.
+    int stid = tid;  // laundered once per tile, see the tile loop
+    auto ch8_of = [&]() __attribute__((always_inline)) { return (stid % G::CPR) * 8; };
     Chunks<F::NL> qst, gst, kst, vst, ost;
     float lse_st = 0.f;
-    // q, k, v rows are laid out like dO and O here (stride W*D between rows, D
-    // between pixels; checked on the host), so one set of offsets serves all five
-    unsigned off[F::NL];
+    // pixel (row, column) of chunk i inside a step
+    auto step_row = [&](int i) __attribute__((always_inline)) { return (stid / G::CPR + i * F::RP) / G::HC; };
+    auto step_col = [&](int i) __attribute__((always_inline)) { return (stid / G::CPR + i * F::RP) % G::HC; };
+    // NR (a compile-time constant: BR, or HR - BR for the rest of a whole block) rows
+    // from y0 on, HC columns from bc on, of one image; positions outside the image
+    // take the nearest pixel.  The offsets are formed anew for every tensor: kept,
+    // they would hold registers through the math of a whole tile.
+    auto fetch = [&](Chunks<F::NL> &reg, const short *img, int y0, int bc, auto nr)
+                     __attribute__((always_inline)) {
+        constexpr int NR = decltype(nr)::value;
+        const char *base = reinterpret_cast<const char *>(img);
 #pragma unroll
-    for (int i = 0; i < F::NL; i++) {
-        const int row = min(srow + i * F::RP, G::ZROW - 1);  // tail: harmless duplicate
-        off[i] = ((unsigned)(row / G::HC) * (unsigned)s.W + (unsigned)(row % G::HC)) * (D * 2u) +
-                 (unsigned)ch8 * 2u;
-    }
-    auto fetch = [&](Chunks<F::NL> &reg, const short *origin) __attribute__((always_inline)) {
-        const char *base = reinterpret_cast<const char *>(origin);
-#pragma unroll
-        for (int i = 0; i < F::NL; i++)
-            reg.v[i] = *reinterpret_cast<const u32x4 *>(base + off[i]);
-    };
-    // The loads of a tile are issued in five parts (one tensor each) spread over
-    // the math of the previous tile: a CU only takes so many vector loads at a
-    // time, and a wave that waits at the queue with all of them at once does no
-    // math meanwhile.
-    auto prefetch_part = [&](const Tile &tl, int part) __attribute__((always_inline)) {
-        const int64_t img_tok = ((int64_t)tl.bb * s.N + tl.nn) * s.H * (int64_t)s.W;
-        const int br = tl.r0 - KS / 2, bc = tl.c0 - KS / 2;
-        const int64_t org = ((int64_t)br * s.W + bc) * D;
-        if (part == 0) {
-            fetch(qst, image<short>(a.q, tl) + org);
-            const int id = min(tid, G::ZROW - 1);
-            lse_st = a.lse[img_tok + (int64_t)(br + id / G::HC) * s.W + bc + id % G::HC];
-        } else if (part == 1) {
-            fetch(kst, image<short>(a.k, tl) + org);
-        } else if (part == 2) {
-            fetch(vst, image<short>(a.v, tl) + org);
-        } else if (part == 3) {
-            fetch(gst, static_cast<const short *>(a.d_o) + img_tok * D + org);
-        } else {
-            fetch(ost, static_cast<const short *>(a.o) + img_tok * D + org);
+        for (int i = 0; i < (NR * G::HC + F::RP - 1) / F::RP; i++) {
+            if ((i + 1) * F::RP <= NR * G::HC || stid / G::CPR + i * F::RP < NR * G::HC) {
+                const int y = min(max(y0 + step_row(i), 0), s.H - 1);
+                const int x = min(max(bc + step_col(i), 0), s.W - 1);
+                const unsigned off =
+                    ((unsigned)y * (unsigned)s.W + (unsigned)x) * (D * 2u) + (unsigned)ch8_of() * 2u;
+                reg.v[i] = *reinterpret_cast<const u32x4 *>(base + off);
+            }
         }
     };
-    auto commit = [&]() __attribute__((always_inline)) {
+    // The loads of a step are issued in five parts (one tensor each) spread over the
+    // math of the current tile: a CU only takes so many vector loads at a time, and a
+    // wave that waits at the queue with all of them at once does no math meanwhile.
+    auto fetch_part = [&](const Tile &tl, int part, int y0, int bc, auto nr)
+                          __attribute__((always_inline)) {
+        constexpr int NR = decltype(nr)::value;
+        const int64_t img_tok = ((int64_t)tl.bb * s.N + tl.nn) * s.H * (int64_t)s.W;
+        if (part == 0) {
+            fetch(qst, image<short>(a.q, tl), y0, bc, nr);
+            const int id = min(stid, NR * G::HC - 1);
+            const int y = min(max(y0 + id / G::HC, 0), s.H - 1), x = min(max(bc + id % G::HC, 0), s.W - 1);
+            lse_st = a.lse[img_tok + (int64_t)y * s.W + x];
+        } else if (part == 1) {
+            fetch(kst, image<short>(a.k, tl), y0, bc, nr);
+        } else if (part == 2) {
+            fetch(vst, image<short>(a.v, tl), y0, bc, nr);
+        } else if (part == 3) {
+            fetch(gst, static_cast<const short *>(a.d_o) + img_tok * D, y0, bc, nr);
+        } else {
+            fetch(ost, static_cast<const short *>(a.o) + img_tok * D, y0, bc, nr);
+        }
+    };
+    // registers -> LDS; image row y goes to row slot (y + HALF) % HR
+    auto commit = [&](int y0, auto nr) __attribute__((always_inline)) {
+        constexpr int NR = decltype(nr)::value;
+        const int s0 = (y0 + HALF) % G::HR;
+        auto lds_row = [&](int pr, int pc) __attribute__((always_inline)) {
+            int slot = s0 + pr;
+            slot = slot >= G::HR ? slot - G::HR : slot;
+            return slot * G::HC + pc;
+        };
 #pragma unroll
-        for (int i = 0; i < F::NL; i++) {
-            const int row = srow + i * F::RP;
+        for (int i = 0; i < (NR * G::HC + F::RP - 1) / F::RP; i++) {
             const float d = group_sum<G::CPR>(dot8<BF>(gst.v[i], ost.v[i]));
-            if (row < G::ZROW) {
-                const int e = row * G::PITCH + ch8;
+            if ((i + 1) * F::RP <= NR * G::HC || stid / G::CPR + i * F::RP < NR * G::HC) {
+                const int row = lds_row(step_row(i), step_col(i));
+                const int e = row * G::PITCH + ch8_of();
                 *reinterpret_cast<u32x4 *>(lds_q + e) = qst.v[i];
                 *reinterpret_cast<u32x4 *>(lds_g + e) = gst.v[i];
                 *reinterpret_cast<u32x4 *>(lds_k + e) = kst.v[i];
                 *reinterpret_cast<u32x4 *>(lds_v + e) = vst.v[i];
-                if (ch8 == 0) lds_stat[row].y = d;
+                if (ch8_of() == 0) lds_stat[row].y = d;
             }
         }
-        if (tid < G::ZROW) lds_stat[tid].x = lse_st * kLog2e;
+        if (stid < NR * G::HC) lds_stat[lds_row(stid / G::HC, stid % G::HC)].x = lse_st * kLog2e;
     };
-
-    Tile cur = inner_tile(sc.t, ts, s.N);
+    // NR rows at once, not overlapped with anything (first tile of a workgroup, first
+    // tile of a column)
+    auto stage_now = [&](const Tile &tl, int y0, int bc, auto nr) __attribute__((always_inline)) {
 #pragma unroll
-    for (int part = 0; part < 5; part++) prefetch_part(cur, part);
-    for (;;) {
-        commit();
-        __syncthreads();
+        for (int part = 0; part < 5; part++) fetch_part(tl, part, y0, bc, nr);
+        commit(y0, nr);
+    };
+    constexpr std::integral_constant<int, F::BR> kStep{};
+    constexpr std::integral_constant<int, G::HR - F::BR> kRest{};
 
-        const int tn = sc.t + sc.step;
+    Tile cur = tile_of_cm(sc.t, ts.tiles_r, ts.tiles_c, s.N);
+    stage_now(cur, cur.r0 - HALF, cur.c0 - HALF, kStep);
+    stage_now(cur, cur.r0 - HALF + F::BR, cur.c0 - HALF, kRest);
+    __syncthreads();
+    const int n = l & 15, g = l >> 4;
+    static_assert(G::SWC == 8 && G::SW == 8 && G::NK == G::NKP,
+                  "the token -> LDS row arithmetic below is written for an 8x8 wave halo");
+    for (;;) {
+        // The thread number is laundered once per tile: the staging arithmetic that is
+        // derived from it would otherwise be hoisted out of the loop and held in
+        // registers that are not there.
+        stid = tid;
+        asm volatile("" : "+v"(stid));
+        const int tn = sc.t + 1;
         const bool more = tn < sc.t_end;
-        const Tile nxt = more ? inner_tile(tn, ts, s.N) : cur;
+        const Tile nxt = more ? tile_of_cm(tn, ts.tiles_r, ts.tiles_c, s.N) : cur;
+        // the tile below in the same image: its block shares k-1 rows with this one
+        const bool below = more && nxt.bb == cur.bb && nxt.nn == cur.nn && nxt.c0 == cur.c0 &&
+                           nxt.r0 == cur.r0 + 8;
+        const int ny0 = below ? cur.r0 - HALF + G::HR : nxt.r0 - HALF;
+        const int nbc = nxt.c0 - HALF;
         auto issue = [&](int part) __attribute__((always_inline)) {
             __builtin_amdgcn_sched_barrier(0);
-            if (more) prefetch_part(nxt, part);
+            if (more) fetch_part(nxt, part, ny0, nbc, kStep);
             __builtin_amdgcn_sched_barrier(0);
         };
-        const int pr = cur.r0 + orow + (n >> 2), pc = cur.c0 + ocol + (n & 3);
-        const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + pr) * s.W + pc;
+
+        const int br = cur.r0 - HALF, bc = cur.c0 - HALF;
+        const int rot = cur.r0 % G::HR;  // row slot of block row 0
+        // LDS row of block position (r, c)
+        auto block_row = [&](int r, int c) __attribute__((always_inline)) {
+            int x = r + rot;
+            x = x >= G::HR ? x - G::HR : x;
+            return x * G::HC + c;
+        };
+        // Tokens of a wave's 8x8 halo with origin (orow, ocol) in the block: token
+        // number tk is halo row tk / 8, column tk % 8.  All token numbers used below
+        // have the form 8 * (a + bit) + c with a a compile-time even number, bit one
+        // lane bit and c < 8, so the LDS row is one of two per-wave (scalar) row-slot
+        // offsets plus a lane column: two or three vector instructions per address.
+        int slot_of[G::SW];
+        auto set_slots = [&](int orow) __attribute__((always_inline)) {
+#pragma unroll
+            for (int j = 0; j < G::SW; j++) {
+                int x = orow + j + rot;
+                x = x >= G::HR ? x - G::HR : x;
+                slot_of[j] = x * G::HC;
+            }
+        };
+        auto tok_row = [&](int a, int bit, int col) __attribute__((always_inline)) {
+            return (bit ? slot_of[a + 1] : slot_of[a]) + col;
+        };
+        // this lane's pixel (query or key)
+        const int py = cur.r0 + (w >> 1) * 4 + (n >> 2), px = cur.c0 + (w & 1) * 4 + (n & 3);
+        const int prow = block_row(py - br, px - bc);
+        auto out_token = [&]() __attribute__((always_inline)) {
+            return (((int64_t)cur.bb * s.N + cur.nn) * s.H + py) * s.W + px;
+        };
+        const int tr = cur.r0 >> 3, tc = cur.c0 >> 3;
+        const bool inner = tr >= ts.ir0 && tr < ts.ir0 + ts.ni_r && tc >= ts.ic0 && tc < ts.ic0 + ts.ni_c;
+
         if (role == 0) {
-            // ---- query side: this lane's query is column n of every product
+            // ---- query side: this lane's query is column n of every product.  The
+            // wave's keys are the (4+k-1)^2 pixels from the window start of its first
+            // query row / column on.
+            const int wy0 = cur.r0 + (w >> 1) * 4, wx0 = cur.c0 + (w & 1) * 4;
+            const int sy0 = win_start(wy0, s.H, KS), sx0 = win_start(wx0, s.W, KS);
+            const int orow = sy0 - br, ocol = sx0 - bc;
+            const int dr = win_start(py, s.H, KS) - sy0, dc = win_start(px, s.W, KS) - sx0;
+            set_slots(orow);
             s16x8 qreg[G::DS], greg[G::DS];
 #pragma unroll
             for (int ds = 0; ds < G::DS; ds++) {
@@ -198,7 +325,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
                 if (mt < 4) issue(mt);
-                const int row = row_of(mt * 16 + n);
+                const int row = tok_row(2 * mt, n >> 3, ocol + (n & 7));
                 const short *kp = lds_k + row * G::PITCH + g * 8;
                 const short *vp = lds_v + row * G::PITCH + g * 8;
                 f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
@@ -209,10 +336,9 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int tk = mt * 16 + g * 4 + i;  // key of accumulator row g*4+i
-                    const bool ok = tk < G::NK &&
-                                    (unsigned)(tk / G::SWC - (n >> 2)) < (unsigned)KS &&
-                                    (unsigned)(tk % G::SWC - (n & 3)) < (unsigned)KS;
+                    // key of accumulator row g*4+i: halo row 2*mt + g/2, column 4*(g%2) + i
+                    const bool ok = ((unsigned)(2 * mt + (g >> 1) - dr) < (unsigned)KS) &
+                                    ((unsigned)(4 * (g & 1) + i - dc) < (unsigned)KS);
                     const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - lse2 : -INFINITY);
                     dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - delta));
                 }
@@ -226,7 +352,8 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 const short *kp[2];
 #pragma unroll
                 for (int h = 0; h < 2; h++)
-                    kp[h] = lds_k + row_of(ks * 32 + h * 16 + g * 4 + (n >> 2)) * G::PITCH +
+                    kp[h] = lds_k +
+                            tok_row(4 * ks + 2 * h, g >> 1, ocol + 4 * (g & 1) + (n >> 2)) * G::PITCH +
                             (n & 3) * (D / 4);
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++)
@@ -234,7 +361,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                         cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)), dsb[ks],
                         dq[mt]);
             }
-            short *dqp = static_cast<short *>(a.dq) + tok * D + g * (D / 4);
+            short *dqp = static_cast<short *>(a.dq) + out_token() * D + g * (D / 4);
 #pragma unroll
             for (int j = 0; j < G::DT / 2; j++) {
                 s16x8 wq;
@@ -245,93 +372,222 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 }
                 *reinterpret_cast<s16x8 *>(dqp + j * 8) = wq;
             }
-            if (g == 0) a.delta[tok] = delta;  // the passes over the border tiles read it
         } else {
-            // ---- key side: this lane's key is column n of every product.  P and dS
-            // of all the halo's queries first, then dV and dK one after the other:
-            // one accumulator at a time leaves the registers to the next tile's halo.
-            s16x8 pb[G::KSTEPS], dsb[G::KSTEPS];
-            {
-                s16x8 kreg[G::DS], vreg[G::DS];
+            // ---- key side: this lane's key is column n of every product
+            if (inner) {
+                // Every window is centred: the queries are the (4+k-1)^2 pixels around
+                // the wave's keys and the mask depends on the lane only.  P and dS of all
+                // of them first, then dV and dK one after the other: one accumulator at a
+                // time leaves the registers to the next tile's rows.
+                const int ocol = (w & 1) * 4;
+                set_slots((w >> 1) * 4);
+                const int kyl = n >> 2, kxl = n & 3;
+                s16x8 pb[G::KSTEPS], dsb[G::KSTEPS];
+                {
+                    // the key row stays in registers; the value row is read where it is
+                    // used (both do not fit beside the next tile's rows)
+                    s16x8 kreg[G::DS];
 #pragma unroll
-                for (int ds = 0; ds < G::DS; ds++) {
-                    kreg[ds] = *reinterpret_cast<const s16x8 *>(lds_k + prow * G::PITCH + ds * 32 + g * 8);
-                    vreg[ds] = *reinterpret_cast<const s16x8 *>(lds_v + prow * G::PITCH + ds * 32 + g * 8);
+                    for (int ds = 0; ds < G::DS; ds++)
+                        kreg[ds] = *reinterpret_cast<const s16x8 *>(lds_k + prow * G::PITCH + ds * 32 + g * 8);
+                    int voff = prow * G::PITCH + g * 8;
+#pragma unroll
+                    for (int mt = 0; mt < G::MT; mt++) {
+                        if (mt < 4) issue(mt);
+                        asm volatile("" : "+v"(voff));  // keep its reads where they are
+                        const short *vrow = lds_v + voff;
+                        const int row = tok_row(2 * mt, n >> 3, ocol + (n & 7));
+                        const short *qp = lds_q + row * G::PITCH + g * 8;
+                        const short *gp = lds_g + row * G::PITCH + g * 8;
+                        f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int ds = 0; ds < G::DS; ds++) {
+                            cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32), kreg[ds], cs);
+                            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32),
+                                            *reinterpret_cast<const s16x8 *>(vrow + ds * 32), cp);
+                        }
+                        // queries of accumulator rows g*4 .. g*4+3: halo row 2*mt + g/2,
+                        // columns 4*(g%2) .. +3, i.e. four consecutive LDS rows
+                        const float2 *stp = lds_stat + tok_row(2 * mt, g >> 1, ocol + 4 * (g & 1));
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const float2 st = stp[i];
+                            const bool ok = ((unsigned)(2 * mt + (g >> 1) - kyl) < (unsigned)KS) &
+                                            ((unsigned)(4 * (g & 1) + i - kxl) < (unsigned)KS);
+                            const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
+                            pb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p);
+                            dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
+                        }
+                    }
                 }
+                issue(4);
+                const int64_t tok = out_token();
+                auto second = [&](const short *lds_x, const s16x8 (&b)[G::KSTEPS], void *out, float mul)
+                                  __attribute__((always_inline)) {
+                    f32x4 acc[G::DT];
 #pragma unroll
-                for (int mt = 0; mt < G::MT; mt++) {
-                    if (mt < 4) issue(mt);
-                    const int row = row_of(mt * 16 + n);
-                    const short *qp = lds_q + row * G::PITCH + g * 8;
-                    const short *gp = lds_g + row * G::PITCH + g * 8;
-                    f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
+                    for (int mt = 0; mt < G::DT; mt++) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int ds = 0; ds < G::DS; ds++) {
-                        cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32), kreg[ds], cs);
-                        cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32), vreg[ds], cp);
+                    for (int ks = 0; ks < G::KSTEPS; ks++) {
+                        const short *xt[2];
+#pragma unroll
+                        for (int h = 0; h < 2; h++)
+                            xt[h] = lds_x +
+                                    tok_row(4 * ks + 2 * h, g >> 1, ocol + 4 * (g & 1) + (n >> 2)) *
+                                        G::PITCH +
+                                    (n & 3) * (D / 4);
+#pragma unroll
+                        for (int mt = 0; mt < G::DT; mt++)
+                            acc[mt] = mfma16<BF>(
+                                cat(lds_read_tr(xt[0] + mt * 4), lds_read_tr(xt[1] + mt * 4)), b[ks],
+                                acc[mt]);
+                    }
+                    short *op = static_cast<short *>(out) + tok * D + g * (D / 4);
+#pragma unroll
+                    for (int j = 0; j < G::DT / 2; j++) {
+                        s16x8 wv;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            wv[i] = cvt16<BF>(acc[2 * j][i] * mul);
+                            wv[4 + i] = cvt16<BF>(acc[2 * j + 1][i] * mul);
+                        }
+                        *reinterpret_cast<s16x8 *>(op + j * 8) = wv;
+                    }
+                };
+                second(lds_g, pb, a.dv, 1.f);
+                second(lds_q, dsb, a.dk, s.scale);
+            } else {
+                // ---- key side of a tile beside the border.  The clamped windows make the
+                // set of queries that attend to the wave's 4x4 keys wider, up to SW + k/2
+                // per axis, and the relation depends on where a query's window starts:
+                // walk a (SW + k/2)^2 region, numbered 16 per row, 32 queries at a time,
+                // with one bit per region row / column telling whether that query row /
+                // column attends this lane's key row / column.  The loop is rolled
+                // (unrolled, the addresses of the whole region would be formed up front).
+                const int ky0 = cur.r0 + (w >> 1) * 4, kx0 = cur.c0 + (w & 1) * 4;
+                constexpr int side = F::SWB;  // region side
+                constexpr int nks = F::KSB;   // reduction steps of 32 queries
+                const int orow = min(max(inv_lo(ky0, KS) - br, 0), G::HR - F::SWB);
+                const int ocol = min(max(inv_lo(kx0, KS) - bc, 0), G::HC - F::SWB);
+                unsigned rmask = 0, cmask = 0;
+#pragma unroll
+                for (int r = 0; r < F::SWB; r++) {
+                    const int qy = br + orow + r, qx = bc + ocol + r;
+                    const bool oky = (r < side) & ((unsigned)qy < (unsigned)s.H) &
+                                     ((unsigned)(py - win_start(qy, s.H, KS)) < (unsigned)KS);
+                    const bool okx = (r < side) & ((unsigned)qx < (unsigned)s.W) &
+                                     ((unsigned)(px - win_start(qx, s.W, KS)) < (unsigned)KS);
+                    rmask |= (oky ? 1u : 0u) << r;
+                    cmask |= (okx ? 1u : 0u) << r;
+                }
+                // region (row, column) of query number tk
+                auto reg_r = [&](int tk) __attribute__((always_inline)) { return tk >> 4; };
+                auto reg_c = [&](int tk) __attribute__((always_inline)) { return tk & 15; };
+                auto row_of = [&](int tk) __attribute__((always_inline)) {
+                    const int r = reg_r(tk), c = reg_c(tk);
+                    return ((r < side) & (c < side)) ? block_row(orow + r, ocol + c) : (int)G::ZROW;
+                };
+                auto ok_of = [&](int tk) __attribute__((always_inline)) {
+                    return ((rmask >> reg_r(tk)) & (cmask >> reg_c(tk)) & 1u) != 0u;
+                };
+                // this lane's key and value rows are read from LDS where they are used
+                // (the registers do not hold them beside the two accumulators and the
+                // next tile's rows)
+                int kvoff = prow * G::PITCH + g * 8;
+                f32x4 dk[G::DT], dv[G::DT];
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++) {
+                    dk[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    dv[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+                // (the next step's loads are issued around the loop, not in it: inside a
+                // rolled loop their destination registers would have to be copied, which
+                // means waiting for them)
+                issue(0);
+                issue(1);
+#pragma unroll 1
+                for (int ks = 0; ks < nks; ks++) {
+                    asm volatile("" : "+v"(kvoff));  // keep their reads in the loop
+                    const short *krow = lds_k + kvoff, *vrow = lds_v + kvoff;
+                    s16x8 pb, dsb;
+#pragma unroll
+                    for (int m2 = 0; m2 < 2; m2++) {
+                        const int mt = ks * 2 + m2;
+                        const int row = row_of(mt * 16 + n);
+                        const short *qp = lds_q + row * G::PITCH + g * 8;
+                        const short *gp = lds_g + row * G::PITCH + g * 8;
+                        f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int ds = 0; ds < G::DS; ds++) {
+                            cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32),
+                                        *reinterpret_cast<const s16x8 *>(krow + ds * 32), cs);
+                            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32),
+                                            *reinterpret_cast<const s16x8 *>(vrow + ds * 32), cp);
+                        }
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const int tk = mt * 16 + g * 4 + i;  // query of accumulator row g*4+i
+                            const float2 st = lds_stat[row_of(tk)];
+                            const float p = __builtin_amdgcn_exp2f(ok_of(tk) ? cs[i] * sc2 - st.x : -INFINITY);
+                            pb[m2 * 4 + i] = cvt16<BF>(p);
+                            dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
+                        }
+                    }
+                    const short *qt[2], *gt[2];
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const int row = row_of(ks * 32 + h * 16 + g * 4 + (n >> 2));
+                        qt[h] = lds_q + row * G::PITCH + (n & 3) * (D / 4);
+                        gt[h] = lds_g + row * G::PITCH + (n & 3) * (D / 4);
                     }
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int tk = mt * 16 + g * 4 + i;  // query of accumulator row g*4+i
-                        const float2 st = lds_stat[row_of(tk)];
-                        const bool ok = tk < G::NK &&
-                                        (unsigned)(tk / G::SWC - (n >> 2)) < (unsigned)KS &&
-                                        (unsigned)(tk % G::SWC - (n & 3)) < (unsigned)KS;
-                        const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
-                        pb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p);
-                        dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
+                    for (int mt = 0; mt < G::DT; mt++) {
+                        dv[mt] = mfma16<BF>(cat(lds_read_tr(gt[0] + mt * 4), lds_read_tr(gt[1] + mt * 4)),
+                                            pb, dv[mt]);
+                        dk[mt] = mfma16<BF>(cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)),
+                                            dsb, dk[mt]);
                     }
                 }
-            }
-            auto second = [&](const short *lds_x, const s16x8 (&b)[G::KSTEPS], void *out, float mul)
-                              __attribute__((always_inline)) {
-                f32x4 acc[G::DT];
-#pragma unroll
-                for (int mt = 0; mt < G::DT; mt++) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int ks = 0; ks < G::KSTEPS; ks++) {
-                    const short *xt[2];
-#pragma unroll
-                    for (int h = 0; h < 2; h++)
-                        xt[h] = lds_x + row_of(ks * 32 + h * 16 + g * 4 + (n >> 2)) * G::PITCH +
-                                (n & 3) * (D / 4);
-#pragma unroll
-                    for (int mt = 0; mt < G::DT; mt++)
-                        acc[mt] = mfma16<BF>(
-                            cat(lds_read_tr(xt[0] + mt * 4), lds_read_tr(xt[1] + mt * 4)), b[ks],
-                            acc[mt]);
-                }
-                short *op = static_cast<short *>(out) + tok * D + g * (D / 4);
+                issue(2);
+                issue(3);
+                issue(4);
+                const int64_t tok = out_token();
+                short *dkp = static_cast<short *>(a.dk) + tok * D + g * (D / 4);
+                short *dvp = static_cast<short *>(a.dv) + tok * D + g * (D / 4);
 #pragma unroll
                 for (int j = 0; j < G::DT / 2; j++) {
-                    s16x8 wv;
+                    s16x8 wk, wv;
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        wv[i] = cvt16<BF>(acc[2 * j][i] * mul);
-                        wv[4 + i] = cvt16<BF>(acc[2 * j + 1][i] * mul);
+                        wk[i] = cvt16<BF>(dk[2 * j][i] * s.scale);
+                        wk[4 + i] = cvt16<BF>(dk[2 * j + 1][i] * s.scale);
+                        wv[i] = cvt16<BF>(dv[2 * j][i]);
+                        wv[4 + i] = cvt16<BF>(dv[2 * j + 1][i]);
                     }
-                    *reinterpret_cast<s16x8 *>(op + j * 8) = wv;
+                    *reinterpret_cast<s16x8 *>(dkp + j * 8) = wk;
+                    *reinterpret_cast<s16x8 *>(dvp + j * 8) = wv;
                 }
-            };
-            issue(4);
-            second(lds_g, pb, a.dv, 1.f);
-            second(lds_q, dsb, a.dk, s.scale);
+            }
         }
+
         if (!more) break;
         __syncthreads();  // every wave is done with this tile's LDS
+        commit(ny0, kStep);
+        if (!below) stage_now(nxt, ny0 + F::BR, nbc, kRest);
+        __syncthreads();
         cur = nxt;
         sc.t = tn;
     }
 }
 
 template <bool BF, int D, int KS>
-int fused_launch(const BwdArgs &a, const TileSet &ts, int64_t n_inner, hipStream_t st) {
+int fused_launch(const BwdArgs &a, const TileSet &ts, int64_t ntiles, hipStream_t st) {
     if constexpr (FGeo<D, KS>::FITS) {
-        const int64_t per_xcd = (n_inner + 7) / 8;
+        const int64_t per_xcd = (ntiles + 7) / 8;
         const int grid = (int)(8 * (per_xcd < 32 ? per_xcd : 32));  // one workgroup per CU
         ProfScope prof(ENATTEN_KERNEL_BWD_FUSED, "bwd_fused_mfma", st);
         hipLaunchKernelGGL((bwd_fused_mfma<BF, D, KS>), dim3(grid), dim3(512), 0, st, a, ts,
-                           (int)n_inner);
+                           (int)ntiles);
         return ENATTEN_OK;
     } else {
         return ENATTEN_EUNSUPPORTED;
@@ -340,17 +596,23 @@ int fused_launch(const BwdArgs &a, const TileSet &ts, int64_t n_inner, hipStream
 
 }  // namespace
 
-bool fused_bwd_supported(int D, int ks) {
-    return D == 128 && ks == 5;
+// The fused backward is built for head_dim 128 with kernel_size 5.  It needs image
+// sides that are multiples of 8 (then the block of a tile holds everything the tile
+// needs, also beside the border), q, k, v rows laid out like dO's, and 32-bit byte
+// offsets inside one image.
+bool fused_bwd_supported(const BwdArgs &a) {
+    auto rows_like_o = [&](const View &v) { return v.sh == (int64_t)a.s.W * a.s.D && v.sw == a.s.D; };
+    return a.s.D == 128 && a.s.kh == 5 && a.s.kw == 5 && a.s.H % 8 == 0 && a.s.W % 8 == 0 &&
+           rows_like_o(a.q) && rows_like_o(a.k) && rows_like_o(a.v) &&
+           (int64_t)a.s.H * a.s.W * a.s.D < ((int64_t)1 << 30);
 }
 
-// dQ, dK, dV of the inner tiles of `ts` (and delta of their queries, for the
-// passes that serve the border tiles).
-int launch_bwd_fused_inner(const BwdArgs &a, bool bf16, const TileSet &ts, int64_t n_inner,
-                           hipStream_t st) {
+// dQ, dK, dV of all tiles in one launch.
+int launch_bwd_fused(const BwdArgs &a, bool bf16, const TileSet &ts, int64_t ntiles,
+                     hipStream_t st) {
     if (a.s.D == 128 && a.s.kh == 5) {
-        if (bf16) return fused_launch<true, 128, 5>(a, ts, n_inner, st);
-        return fused_launch<false, 128, 5>(a, ts, n_inner, st);
+        if (bf16) return fused_launch<true, 128, 5>(a, ts, ntiles, st);
+        return fused_launch<false, 128, 5>(a, ts, ntiles, st);
     }
     return ENATTEN_EUNSUPPORTED;
 }
