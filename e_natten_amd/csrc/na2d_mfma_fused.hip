@@ -75,6 +75,12 @@ __device__ __forceinline__ float dot8(u32x4 a, u32x4 b) {
     }
     return even + odd;
 }
+// ok ? x : -inf as bit arithmetic.  Written as a conditional expression, the compiler
+// moves the LDS read that feeds x under a branch on ok (one branch per logit).
+__device__ __forceinline__ float keep_or_ninf(float x, bool ok) {
+    const int m = ok ? -1 : 0;
+    return __int_as_float((__float_as_int(x) & m) | ((int)0xff800000 & ~m));
+}
 // sum over aligned groups of LANES (4, 8 or 16) consecutive lanes, in every lane
 template <int LANES>
 __device__ __forceinline__ float group_sum(float x) {
@@ -414,7 +420,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                             const float2 st = stp[i];
                             const bool ok = ((unsigned)(2 * mt + (g >> 1) - kyl) < (unsigned)KS) &
                                             ((unsigned)(4 * (g & 1) + i - kxl) < (unsigned)KS);
-                            const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
+                            const float p = __builtin_amdgcn_exp2f(keep_or_ninf(cs[i] * sc2 - st.x, ok));
                             pb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p);
                             dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
                         }
@@ -528,7 +534,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                         for (int i = 0; i < 4; i++) {
                             const int tk = mt * 16 + g * 4 + i;  // query of accumulator row g*4+i
                             const float2 st = lds_stat[row_of(tk)];
-                            const float p = __builtin_amdgcn_exp2f(ok_of(tk) ? cs[i] * sc2 - st.x : -INFINITY);
+                            const float p = __builtin_amdgcn_exp2f(keep_or_ninf(cs[i] * sc2 - st.x, ok_of(tk)));
                             pb[m2 * 4 + i] = cvt16<BF>(p);
                             dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
                         }

@@ -64,12 +64,14 @@ def test_config2_bf16_readme_shape(side, path):
     _case((4, 4, side, side, 128), BF, 5, what="C2 side %d" % side)
 
 
-@pytest.mark.parametrize("shape,dtype", [((4, 4, 32, 32, 128), BF), ((2, 2, 64, 64, 128), BF),
+@pytest.mark.parametrize("shape,dtype", [((1, 1, 8, 8, 128), BF), ((1, 2, 16, 24, 128), BF),
+                                         ((4, 4, 32, 32, 128), BF), ((2, 3, 64, 40, 128), BF),
                                          ((4, 4, 128, 128, 128), BF), ((1, 3, 40, 72, 128), F16),
                                          ((1, 2, 37, 50, 128), BF)])
 def test_fused_backward_path(shape, dtype, _lib):
-    # the opt-in fused backward (inner tiles: dQ, dK, dV from one staging; border
-    # tiles: the two-pass kernels) against the oracle, square, ragged and fp16
+    # the opt-in fused backward (dQ, dK, dV of every tile from one staging of q, k, v,
+    # dO) against the oracle: images that are all border, mixed, fp16; the last shape
+    # has sides that are no multiples of 8 and is served by the two-pass kernels
     from e_natten_amd._lib import PATH_MFMA_FUSED
     prev = _lib.enatten_set_path(PATH_MFMA_FUSED)
     try:
