@@ -24,7 +24,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TF = 2500.0   # dense bf16, published
-KERNELS = ("fwd", "bwd_dq", "bwd_dkdv")
+KERNELS = ("fwd", "bwd_dq", "bwd_dkdv", "bwd_fused")
 
 
 def algorithmic_bytes(B, N, H, W, D, esize):
@@ -32,11 +32,12 @@ def algorithmic_bytes(B, N, H, W, D, esize):
     fwd : read q,k,v, write o (+ 4 B/query log-sum-exp)
     dq  : read q,k,v,dO (+ lse), write dq
     dkdv: read q,k,v,dO (+ lse), write dk,dv
+    fused backward (opt-in): read q,k,v,dO (+ lse), write dq,dk,dv
     path: 11*M*s + 8*q, the fused-backward minimum (q,k,v,dO read once in bwd)."""
     q = B * N * H * W
     M = q * D * esize
     return {"fwd": 4 * M + 4 * q, "bwd_dq": 5 * M + 4 * q, "bwd_dkdv": 6 * M + 4 * q,
-            "path": 11 * M + 8 * q}
+            "bwd_fused": 7 * M + 4 * q, "path": 11 * M + 8 * q}
 
 
 def cpu_baseline(shape, ks, dtype, useful_flop, budget_rows=8):
@@ -124,7 +125,7 @@ def run_all_configs():
         torch.cuda.synchronize()
         lib.enatten_profile_enable(0)
         us = []
-        for i in range(3):
+        for i in range(3):  # forward, dQ pass, dK/dV pass (the default backward)
             n, tot = ctypes.c_int(), ctypes.c_double()
             lib.enatten_profile_read(i, ctypes.byref(n), ctypes.byref(tot))
             us.append(tot.value / max(n.value, 1) * 1e3)
@@ -157,6 +158,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-sweep", action="store_true", help="skip the other image sides")
     ap.add_argument("--simt", action="store_true", help="force the vector-ALU kernels")
+    ap.add_argument("--fused-bwd", action="store_true",
+                    help="use the opt-in fused backward kernel where it is built")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run a plain 256 MiB device copy (calibrates rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -177,6 +180,8 @@ def main():
     lib = _lib.load()
     if args.simt:
         lib.enatten_set_path(_lib.PATH_SIMT)
+    elif args.fused_bwd:
+        lib.enatten_set_path(_lib.PATH_MFMA_FUSED)
     dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype]
     B, N, S, D, ks = args.batch, args.heads, args.side, args.head_dim, args.kernel_size
     shape = (B, N, S, S, D)
