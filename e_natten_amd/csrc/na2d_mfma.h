@@ -64,6 +64,68 @@ __device__ __forceinline__ float col_sum(float x) {
     return x + __shfl_xor(x, 32, 64);
 }
 
+// Stores one token's D output channels from the accumulators of the second product.
+// `acc[t][i]` is channel g*D/4 + t*4 + i of this lane's token (lanes l, l+16, l+32,
+// l+48 share a token, g = l/16): D/32 pieces of 16 bytes per lane.  Written as they
+// are, a store instruction would put 16-byte pieces D/2 bytes apart (measured at
+// D = 128: 3.6 TB/s for a pure write stream of that shape against 5.4 TB/s for 64-byte
+// runs).  So at D = 128 the four lanes of a token first exchange pieces with
+// v_permlane*_swap (a 4x4 transpose between lane group g and piece number j), and store
+// j of the four lanes then covers 64 contiguous bytes.  Every lane of the wave
+// must call this; `live` says whether this lane's token exists.
+template <bool BF, int D>
+__device__ __forceinline__ void store_token(short *token, int g, const f32x4 *acc, float mul,
+                                            bool live) {
+    constexpr int NP = D / 32;
+    u32x4 p[NP];
+#pragma unroll
+    for (int j = 0; j < NP; j++) {
+        s16x8 w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[i] = cvt16<BF>(acc[2 * j][i] * mul);
+            w[4 + i] = cvt16<BF>(acc[2 * j + 1][i] * mul);
+        }
+        p[j] = __builtin_bit_cast(u32x4, w);
+    }
+    if constexpr (NP == 4) {
+        typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+        // lanes l and l^32 (g bit 1) exchange pieces j and j^2 ...
+#pragma unroll
+        for (int j0 = 0; j0 < 2; j0++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const u32x2 r = __builtin_amdgcn_permlane32_swap(p[j0][c], p[j0 + 2][c], false, false);
+                p[j0][c] = r[0];
+                p[j0 + 2][c] = r[1];
+            }
+        // ... then lanes l and l^16 (g bit 0) pieces j and j^1
+#pragma unroll
+        for (int j1 = 0; j1 < 2; j1++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const u32x2 r =
+                    __builtin_amdgcn_permlane16_swap(p[2 * j1][c], p[2 * j1 + 1][c], false, false);
+                p[2 * j1][c] = r[0];
+                p[2 * j1 + 1][c] = r[1];
+            }
+        // piece j of this lane is now channels j*D/4 + g*8 .. +8
+        if (live) {
+#pragma unroll
+            for (int j = 0; j < NP; j++)
+                *reinterpret_cast<u32x4 *>(token + j * (D / 4) + g * 8) = p[j];
+        }
+    } else {
+        // D = 32: the four lanes of a token already cover its 64 bytes.  D = 64 (pieces
+        // 32 bytes apart): the corresponding exchange was measured and gains nothing.
+        if (live) {
+#pragma unroll
+            for (int j = 0; j < NP; j++)
+                *reinterpret_cast<u32x4 *>(token + g * (D / 4) + j * 8) = p[j];
+        }
+    }
+}
+
 template <int D, int KS>
 struct Geo {
     static constexpr int TH = 8, TW = 8;          // pixels per workgroup

@@ -166,22 +166,9 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
                         o[mt]);
             }
 
-            if (lq.live) {
-                const float inv = 1.f / sum;
-                short *op = static_cast<short *>(a.o) + lq.tok * D + g * (D / 4);
-#pragma unroll
-                for (int j = 0; j < G::DT / 2; j++) {
-                    s16x8 w;
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        w[i] = cvt16<BF>(o[2 * j][i] * inv);
-                        w[4 + i] = cvt16<BF>(o[2 * j + 1][i] * inv);
-                    }
-                    *reinterpret_cast<s16x8 *>(op + j * 8) = w;
-                }
-                if (a.lse && g == 0)
-                    a.lse[lq.tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
-            }
+            store_token<BF, D>(static_cast<short *>(a.o) + lq.tok * D, g, o, 1.f / sum, lq.live);
+            if (lq.live && a.lse && g == 0)
+                a.lse[lq.tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
         }
 
         if (!more) break;
@@ -360,20 +347,8 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
                         dq[mt]);
             }
 
-            if (lq.live) {
-                short *dqp = static_cast<short *>(a.dq) + lq.tok * D + g * (D / 4);
-#pragma unroll
-                for (int j = 0; j < G::DT / 2; j++) {
-                    s16x8 w;
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        w[i] = cvt16<BF>(dq[2 * j][i] * s.scale);
-                        w[4 + i] = cvt16<BF>(dq[2 * j + 1][i] * s.scale);
-                    }
-                    *reinterpret_cast<s16x8 *>(dqp + j * 8) = w;
-                }
-                if (g == 0) a.delta[lq.tok] = delta;
-            }
+            store_token<BF, D>(static_cast<short *>(a.dq) + lq.tok * D, g, dq, s.scale, lq.live);
+            if (lq.live && g == 0) a.delta[lq.tok] = delta;
         }
 
         if (!more) break;
@@ -588,21 +563,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         {
             const int kr = cur.r0 + orow + (n >> 2), kc = cur.c0 + ocol + (n & 3);
             const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + kr) * s.W + kc;
-            short *dkp = static_cast<short *>(a.dk) + tok * D + g * (D / 4);
-            short *dvp = static_cast<short *>(a.dv) + tok * D + g * (D / 4);
-#pragma unroll
-            for (int j = 0; j < G::DT / 2; j++) {
-                s16x8 wk, wv;
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    wk[i] = cvt16<BF>(dk[2 * j][i] * s.scale);
-                    wk[4 + i] = cvt16<BF>(dk[2 * j + 1][i] * s.scale);
-                    wv[i] = cvt16<BF>(dv[2 * j][i]);
-                    wv[4 + i] = cvt16<BF>(dv[2 * j + 1][i]);
-                }
-                *reinterpret_cast<s16x8 *>(dkp + j * 8) = wk;
-                *reinterpret_cast<s16x8 *>(dvp + j * 8) = wv;
-            }
+            store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
+            store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
         }
 
         if (!more) break;
@@ -777,24 +739,11 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
         }
 
         const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
-        if (cur.last && live) {
+        if (cur.last) {
             const int64_t tok =
                 (((int64_t)cur.tl.bb * s.N + cur.tl.nn) * s.H + kr) * s.W + kc;
-            short *dkp = static_cast<short *>(a.dk) + tok * D + g * (D / 4);
-            short *dvp = static_cast<short *>(a.dv) + tok * D + g * (D / 4);
-#pragma unroll
-            for (int j = 0; j < G::DT / 2; j++) {
-                s16x8 wk, wv;
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    wk[i] = cvt16<BF>(dk[2 * j][i] * s.scale);
-                    wk[4 + i] = cvt16<BF>(dk[2 * j + 1][i] * s.scale);
-                    wv[i] = cvt16<BF>(dv[2 * j][i]);
-                    wv[4 + i] = cvt16<BF>(dv[2 * j + 1][i]);
-                }
-                *reinterpret_cast<s16x8 *>(dkp + j * 8) = wk;
-                *reinterpret_cast<s16x8 *>(dvp + j * 8) = wv;
-            }
+            store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, live);
+            store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, live);
         }
 
         if (!more) break;

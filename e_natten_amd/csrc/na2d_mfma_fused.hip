@@ -367,17 +367,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                         cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)), dsb[ks],
                         dq[mt]);
             }
-            short *dqp = static_cast<short *>(a.dq) + out_token() * D + g * (D / 4);
-#pragma unroll
-            for (int j = 0; j < G::DT / 2; j++) {
-                s16x8 wq;
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    wq[i] = cvt16<BF>(dq[2 * j][i] * s.scale);
-                    wq[4 + i] = cvt16<BF>(dq[2 * j + 1][i] * s.scale);
-                }
-                *reinterpret_cast<s16x8 *>(dqp + j * 8) = wq;
-            }
+            store_token<BF, D>(static_cast<short *>(a.dq) + out_token() * D, g, dq, s.scale, true);
         } else {
             // ---- key side: this lane's key is column n of every product
             if (inner) {
@@ -448,17 +438,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                                 cat(lds_read_tr(xt[0] + mt * 4), lds_read_tr(xt[1] + mt * 4)), b[ks],
                                 acc[mt]);
                     }
-                    short *op = static_cast<short *>(out) + tok * D + g * (D / 4);
-#pragma unroll
-                    for (int j = 0; j < G::DT / 2; j++) {
-                        s16x8 wv;
-#pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            wv[i] = cvt16<BF>(acc[2 * j][i] * mul);
-                            wv[4 + i] = cvt16<BF>(acc[2 * j + 1][i] * mul);
-                        }
-                        *reinterpret_cast<s16x8 *>(op + j * 8) = wv;
-                    }
+                    store_token<BF, D>(static_cast<short *>(out) + tok * D, g, acc, mul, true);
                 };
                 second(lds_g, pb, a.dv, 1.f);
                 second(lds_q, dsb, a.dk, s.scale);
@@ -558,21 +538,8 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 issue(3);
                 issue(4);
                 const int64_t tok = out_token();
-                short *dkp = static_cast<short *>(a.dk) + tok * D + g * (D / 4);
-                short *dvp = static_cast<short *>(a.dv) + tok * D + g * (D / 4);
-#pragma unroll
-                for (int j = 0; j < G::DT / 2; j++) {
-                    s16x8 wk, wv;
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        wk[i] = cvt16<BF>(dk[2 * j][i] * s.scale);
-                        wk[4 + i] = cvt16<BF>(dk[2 * j + 1][i] * s.scale);
-                        wv[i] = cvt16<BF>(dv[2 * j][i]);
-                        wv[4 + i] = cvt16<BF>(dv[2 * j + 1][i]);
-                    }
-                    *reinterpret_cast<s16x8 *>(dkp + j * 8) = wk;
-                    *reinterpret_cast<s16x8 *>(dvp + j * 8) = wv;
-                }
+                store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
+                store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
             }
         }
 
