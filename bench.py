@@ -32,7 +32,7 @@ def algorithmic_bytes(B, N, H, W, D, esize):
     fwd : read q,k,v, write o (+ 4 B/query log-sum-exp)
     dq  : read q,k,v,dO (+ lse), write dq
     dkdv: read q,k,v,dO (+ lse), write dk,dv
-    fused backward (opt-in): read q,k,v,dO (+ lse), write dq,dk,dv
+    fused backward: read q,k,v,dO (+ lse), write dq,dk,dv
     path: 11*M*s + 8*q, the fused-backward minimum (q,k,v,dO read once in bwd)."""
     q = B * N * H * W
     M = q * D * esize
@@ -125,17 +125,17 @@ def run_all_configs():
         torch.cuda.synchronize()
         lib.enatten_profile_enable(0)
         us = []
-        for i in range(3):  # forward, dQ pass, dK/dV pass (the default backward)
+        for i in range(4):  # forward, dQ pass, dK/dV pass, fused backward (one or the other)
             n, tot = ctypes.c_int(), ctypes.c_double()
             lib.enatten_profile_read(i, ctypes.byref(n), ctypes.byref(tot))
-            us.append(tot.value / max(n.value, 1) * 1e3)
+            us.append(tot.value / n.value * 1e3 if n.value else 0.0)
         qn = B * N * S * S
         flop = 14.0 * ks * ks * D * qn
         byt = 11 * qn * D * q.element_size() + 8 * qn
         tot_us = sum(us)
         recs.append({"config": name, "shape": [B, N, S, S, D], "k": ks, "dtype": dt,
                      "path": kernel_path(D, ks, dts[dt]), "fwd_us": us[0], "bwd_dq_us": us[1],
-                     "bwd_dkdv_us": us[2], "kernel_us": tot_us,
+                     "bwd_dkdv_us": us[2], "bwd_fused_us": us[3], "kernel_us": tot_us,
                      "useful_tflops": flop / tot_us / 1e6,
                      "alg_GBps": byt / tot_us / 1e3,
                      "frac_hbm_peak": byt / tot_us / 1e3 / HBM_PEAK_GBS,
@@ -159,7 +159,9 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the other image sides")
     ap.add_argument("--simt", action="store_true", help="force the vector-ALU kernels")
     ap.add_argument("--fused-bwd", action="store_true",
-                    help="use the opt-in fused backward kernel where it is built")
+                    help="force the fused backward kernel wherever it is built")
+    ap.add_argument("--split-bwd", action="store_true",
+                    help="force the two-pass backward (dQ, then dK/dV)")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run a plain 256 MiB device copy (calibrates rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -182,6 +184,8 @@ def main():
         lib.enatten_set_path(_lib.PATH_SIMT)
     elif args.fused_bwd:
         lib.enatten_set_path(_lib.PATH_MFMA_FUSED)
+    elif args.split_bwd:
+        lib.enatten_set_path(_lib.PATH_MFMA_SPLIT)
     dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype]
     B, N, S, D, ks = args.batch, args.heads, args.side, args.head_dim, args.kernel_size
     shape = (B, N, S, S, D)

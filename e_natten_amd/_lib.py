@@ -9,7 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libenatten.so")
 
 F32, BF16, F16 = 0, 1, 2
-PATH_NONE, PATH_SIMT, PATH_MFMA, PATH_MFMA_FUSED = 0, 1, 2, 3
+PATH_NONE, PATH_SIMT, PATH_MFMA, PATH_MFMA_FUSED, PATH_MFMA_SPLIT = 0, 1, 2, 3, 4
 
 _lock = threading.Lock()
 _lib = None

@@ -139,7 +139,8 @@ int enatten2d_kernel_path(int D, int kernel_size, int dtype) {
 }
 
 int enatten_set_path(int path) {
-    if (path != 0 && path != ENATTEN_PATH_SIMT && path != ENATTEN_PATH_MFMA_FUSED)
+    if (path != 0 && path != ENATTEN_PATH_SIMT && path != ENATTEN_PATH_MFMA_FUSED &&
+        path != ENATTEN_PATH_MFMA_SPLIT)
         return g_path.load();
     return g_path.exchange(path);
 }
@@ -194,7 +195,7 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o, co
     a.zinv = a.delta + (size_t)B * heads * H * W;
     a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (use_mfma(D, kernel_size, dtype)) return launch_bwd_mfma(a, dtype, g_path.load() == ENATTEN_PATH_MFMA_FUSED, st);
+    if (use_mfma(D, kernel_size, dtype)) return launch_bwd_mfma(a, dtype, g_path.load(), st);
     return launch_bwd_simt(a, dtype, st);
 }
 

@@ -77,7 +77,9 @@ int launch_bwd_simt(const BwdArgs &a, int dtype, hipStream_t st);
 // matrix-core kernels: bf16 / f16, D in {32, 64, 128}, square odd window
 bool mfma_supported(int D, int ks, int dtype);
 int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st);
-int launch_bwd_mfma(const BwdArgs &a, int dtype, bool allow_fused, hipStream_t st);
+// `path`: 0 chooses between the two-pass and the fused backward, ENATTEN_PATH_MFMA_FUSED /
+// ENATTEN_PATH_MFMA_SPLIT force one of them
+int launch_bwd_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st);
 // fused backward (dQ, dK, dV of every tile from one staging), where built
 bool fused_bwd_supported(const BwdArgs &a);
 int launch_bwd_fused(const BwdArgs &a, bool bf16, const TileSet &ts, int64_t ntiles,

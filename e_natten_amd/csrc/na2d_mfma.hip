@@ -814,7 +814,7 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
 }
 
 template <bool BF, int D, int KS>
-int bwd_launch(const BwdArgs &a, bool allow_fused, hipStream_t st) {
+int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
     if constexpr (fits<D, KS>()) {
         using G = Geo<D, KS>;
         const int tiles_r = (a.s.H + G::TH - 1) / G::TH, tiles_c = (a.s.W + G::TW - 1) / G::TW;
@@ -830,7 +830,12 @@ int bwd_launch(const BwdArgs &a, bool allow_fused, hipStream_t st) {
         const int64_t slabs = (int64_t)a.s.B * a.s.N;
         const int64_t n_inner = slabs * ts.ni_r * ts.ni_c, n_frame = nb - n_inner;
 
-        if (allow_fused && fused_bwd_supported(a)) {
+        // The fused backward where it is built and measured faster than the two passes:
+        // enough tiles for every CU to walk a while, and images large enough that the
+        // tiles beside the border (1.5x the cost of an inner tile there) are few.
+        const bool fused_pays = nb >= 2048 && tiles_r >= 12 && tiles_c >= 12;
+        if (path != ENATTEN_PATH_MFMA_SPLIT && fused_bwd_supported(a) &&
+            (path == ENATTEN_PATH_MFMA_FUSED || fused_pays)) {
             launch_bwd_fused(a, BF, ts, nb, st);
             return check_launch("enatten2d_bwd");
         }
@@ -920,15 +925,15 @@ int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st) {
     return ENATTEN_EUNSUPPORTED;
 }
 
-int launch_bwd_mfma(const BwdArgs &a, int dtype, bool allow_fused, hipStream_t st) {
+int launch_bwd_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st) {
     auto al = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
     if (!layout_ok(a.q) || !layout_ok(a.k) || !layout_ok(a.v) || !al(a.o) || !al(a.d_o) ||
         !al(a.dq) || !al(a.dk) || !al(a.dv))
         return launch_bwd_simt(a, dtype, st);
     if (dtype == ENATTEN_BF16) {
-        ENATTEN_BY_D(bwd_launch, true, a, allow_fused, st)
+        ENATTEN_BY_D(bwd_launch, true, a, path, st)
     } else {
-        ENATTEN_BY_D(bwd_launch, false, a, allow_fused, st)
+        ENATTEN_BY_D(bwd_launch, false, a, path, st)
     }
     set_error("no matrix-core kernel for head_dim %d, kernel_size %d", a.s.D, a.s.kh);
     return ENATTEN_EUNSUPPORTED;

@@ -36,9 +36,16 @@ template <int D, int KS>
 struct FGeo {
     using G = Geo<D, KS>;
     static constexpr int NT = 512;                        // threads per workgroup
-    static constexpr int RP = NT / G::CPR;                // block pixels staged per pass
+    // Staging is shared unevenly: the key side has more arithmetic per tile, so the
+    // query-side waves move five sixths of a step and the key-side waves the rest
+    // (issuing a load blocks a wave for as long as some of its arithmetic takes).
+    static constexpr int RPH = NT / 2 / G::CPR;           // block pixels per pass and side
     static constexpr int BR = 8;                          // block rows staged per step
-    static constexpr int NL = (BR * G::HC + RP - 1) / RP; // passes per step
+    static constexpr int passes(int nrows) { return (nrows * G::HC + RPH - 1) / RPH; }
+    static constexpr int q_passes(int nrows) {
+        return passes(nrows) - (passes(nrows) / 6 > 1 ? passes(nrows) / 6 : 1);
+    }
+    static constexpr int NL = q_passes(BR);               // chunks per thread and tensor (query side)
     // Key side beside the border: the queries that attend to a wave's 4x4 keys
     // span up to SW + k/2 rows and columns there; they are numbered 16 per row.
     static constexpr int SWB = G::SW + KS / 2;
@@ -171,22 +178,34 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     auto ch8_of = [&]() __attribute__((always_inline)) { return (stid % G::CPR) * 8; };
     Chunks<F::NL> qst, gst, kst, vst, ost;
     float lse_st = 0.f;
-    // pixel (row, column) of chunk i inside a step
-    auto step_row = [&](int i) __attribute__((always_inline)) { return (stid / G::CPR + i * F::RP) / G::HC; };
-    auto step_col = [&](int i) __attribute__((always_inline)) { return (stid / G::CPR + i * F::RP) % G::HC; };
+    // Pixel number (row-major inside the step) of chunk i of this thread, or -1: a
+    // step of NR rows has NR*HC pixels; the query-side waves take the first
+    // q_passes(NR) * RPH of them, the key-side waves the rest.
+    auto step_pixel = [&](int i, auto nr, int side) __attribute__((always_inline)) {
+        constexpr int NR = decltype(nr)::value;
+        constexpr int QP = F::q_passes(NR), KP = F::passes(NR) - QP;
+        const int mine = side == 0 ? QP : KP;
+        const int pix = (side == 0 ? 0 : QP * F::RPH) + (stid & (F::NT / 2 - 1)) / G::CPR + i * F::RPH;
+        return (i < mine && pix < NR * G::HC) ? pix : -1;
+    };
     // NR (a compile-time constant: BR, or HR - BR for the rest of a whole block) rows
     // from y0 on, HC columns from bc on, of one image; positions outside the image
     // take the nearest pixel.  The offsets are formed anew for every tensor: kept,
     // they would hold registers through the math of a whole tile.
-    auto fetch = [&](Chunks<F::NL> &reg, const short *img, int y0, int bc, auto nr)
+    // `side` (a compile-time 0 or 1) is the side of the calling wave: the key-side waves
+    // then provably never touch the chunk registers beyond their share.
+    auto fetch = [&](Chunks<F::NL> &reg, const short *img, int y0, int bc, auto nr, auto side)
                      __attribute__((always_inline)) {
         constexpr int NR = decltype(nr)::value;
+        constexpr int SIDE = decltype(side)::value;
+        constexpr int MINE = SIDE == 0 ? F::q_passes(NR) : F::passes(NR) - F::q_passes(NR);
         const char *base = reinterpret_cast<const char *>(img);
 #pragma unroll
-        for (int i = 0; i < (NR * G::HC + F::RP - 1) / F::RP; i++) {
-            if ((i + 1) * F::RP <= NR * G::HC || stid / G::CPR + i * F::RP < NR * G::HC) {
-                const int y = min(max(y0 + step_row(i), 0), s.H - 1);
-                const int x = min(max(bc + step_col(i), 0), s.W - 1);
+        for (int i = 0; i < MINE; i++) {
+            const int pix = step_pixel(i, nr, SIDE);
+            if (pix >= 0) {
+                const int y = min(max(y0 + pix / G::HC, 0), s.H - 1);
+                const int x = min(max(bc + pix % G::HC, 0), s.W - 1);
                 const unsigned off =
                     ((unsigned)y * (unsigned)s.W + (unsigned)x) * (D * 2u) + (unsigned)ch8_of() * 2u;
                 reg.v[i] = *reinterpret_cast<const u32x4 *>(base + off);
@@ -196,23 +215,23 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     // The loads of a step are issued in five parts (one tensor each) spread over the
     // math of the current tile: a CU only takes so many vector loads at a time, and a
     // wave that waits at the queue with all of them at once does no math meanwhile.
-    auto fetch_part = [&](const Tile &tl, int part, int y0, int bc, auto nr)
+    auto fetch_part = [&](const Tile &tl, int part, int y0, int bc, auto nr, auto side)
                           __attribute__((always_inline)) {
         constexpr int NR = decltype(nr)::value;
         const int64_t img_tok = ((int64_t)tl.bb * s.N + tl.nn) * s.H * (int64_t)s.W;
         if (part == 0) {
-            fetch(qst, image<short>(a.q, tl), y0, bc, nr);
+            fetch(qst, image<short>(a.q, tl), y0, bc, nr, side);
             const int id = min(stid, NR * G::HC - 1);
             const int y = min(max(y0 + id / G::HC, 0), s.H - 1), x = min(max(bc + id % G::HC, 0), s.W - 1);
             lse_st = a.lse[img_tok + (int64_t)y * s.W + x];
         } else if (part == 1) {
-            fetch(kst, image<short>(a.k, tl), y0, bc, nr);
+            fetch(kst, image<short>(a.k, tl), y0, bc, nr, side);
         } else if (part == 2) {
-            fetch(vst, image<short>(a.v, tl), y0, bc, nr);
+            fetch(vst, image<short>(a.v, tl), y0, bc, nr, side);
         } else if (part == 3) {
-            fetch(gst, static_cast<const short *>(a.d_o) + img_tok * D, y0, bc, nr);
+            fetch(gst, static_cast<const short *>(a.d_o) + img_tok * D, y0, bc, nr, side);
         } else {
-            fetch(ost, static_cast<const short *>(a.o) + img_tok * D, y0, bc, nr);
+            fetch(ost, static_cast<const short *>(a.o) + img_tok * D, y0, bc, nr, side);
         }
     };
     // registers -> LDS; image row y goes to row slot (y + HALF) % HR
@@ -225,10 +244,11 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
             return slot * G::HC + pc;
         };
 #pragma unroll
-        for (int i = 0; i < (NR * G::HC + F::RP - 1) / F::RP; i++) {
+        for (int i = 0; i < F::q_passes(NR); i++) {
             const float d = group_sum<G::CPR>(dot8<BF>(gst.v[i], ost.v[i]));
-            if ((i + 1) * F::RP <= NR * G::HC || stid / G::CPR + i * F::RP < NR * G::HC) {
-                const int row = lds_row(step_row(i), step_col(i));
+            const int pix = step_pixel(i, nr, role);
+            if (pix >= 0) {
+                const int row = lds_row(pix / G::HC, pix % G::HC);
                 const int e = row * G::PITCH + ch8_of();
                 *reinterpret_cast<u32x4 *>(lds_q + e) = qst.v[i];
                 *reinterpret_cast<u32x4 *>(lds_g + e) = gst.v[i];
@@ -241,9 +261,16 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     };
     // NR rows at once, not overlapped with anything (first tile of a workgroup, first
     // tile of a column)
+    constexpr std::integral_constant<int, 0> kQuerySide{};
+    constexpr std::integral_constant<int, 1> kKeySide{};
     auto stage_now = [&](const Tile &tl, int y0, int bc, auto nr) __attribute__((always_inline)) {
+        if (role == 0) {
 #pragma unroll
-        for (int part = 0; part < 5; part++) fetch_part(tl, part, y0, bc, nr);
+            for (int part = 0; part < 5; part++) fetch_part(tl, part, y0, bc, nr, kQuerySide);
+        } else {
+#pragma unroll
+            for (int part = 0; part < 5; part++) fetch_part(tl, part, y0, bc, nr, kKeySide);
+        }
         commit(y0, nr);
     };
     constexpr std::integral_constant<int, F::BR> kStep{};
@@ -262,6 +289,16 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         // registers that are not there.
         stid = tid;
         asm volatile("" : "+v"(stid));
+        // The staging registers carry nothing from one tile to the next (they are
+        // filled during a tile and written to LDS at its end): start every tile with
+        // fresh ones, or the chunks that only the query side fills would count as
+        // live through the key side's arithmetic.
+        {
+            Chunks<F::NL> fresh;
+#pragma unroll
+            for (int i = 0; i < F::NL; i++) asm volatile("" : "=v"(fresh.v[i]));
+            qst = fresh; gst = fresh; kst = fresh; vst = fresh; ost = fresh;
+        }
         const int tn = sc.t + 1;
         const bool more = tn < sc.t_end;
         const Tile nxt = more ? tile_of_cm(tn, ts.tiles_r, ts.tiles_c, s.N) : cur;
@@ -270,9 +307,9 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                            nxt.r0 == cur.r0 + 8;
         const int ny0 = below ? cur.r0 - HALF + G::HR : nxt.r0 - HALF;
         const int nbc = nxt.c0 - HALF;
-        auto issue = [&](int part) __attribute__((always_inline)) {
+        auto issue_as = [&](int part, auto side) __attribute__((always_inline)) {
             __builtin_amdgcn_sched_barrier(0);
-            if (more) fetch_part(nxt, part, ny0, nbc, kStep);
+            if (more) fetch_part(nxt, part, ny0, nbc, kStep, side);
             __builtin_amdgcn_sched_barrier(0);
         };
 
@@ -311,6 +348,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         const bool inner = tr >= ts.ir0 && tr < ts.ir0 + ts.ni_r && tc >= ts.ic0 && tc < ts.ic0 + ts.ni_c;
 
         if (role == 0) {
+            auto issue = [&](int part) __attribute__((always_inline)) { issue_as(part, kQuerySide); };
             // ---- query side: this lane's query is column n of every product.  The
             // wave's keys are the (4+k-1)^2 pixels from the window start of its first
             // query row / column on.
@@ -369,6 +407,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
             }
             store_token<BF, D>(static_cast<short *>(a.dq) + out_token() * D, g, dq, s.scale, true);
         } else {
+            auto issue = [&](int part) __attribute__((always_inline)) { issue_as(part, kKeySide); };
             // ---- key side: this lane's key is column n of every product
             if (inner) {
                 // Every window is centred: the queries are the (4+k-1)^2 pixels around
@@ -380,18 +419,15 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 const int kyl = n >> 2, kxl = n & 3;
                 s16x8 pb[G::KSTEPS], dsb[G::KSTEPS];
                 {
-                    // the key row stays in registers; the value row is read where it is
-                    // used (both do not fit beside the next tile's rows)
-                    s16x8 kreg[G::DS];
+                    s16x8 kreg[G::DS], vreg[G::DS];
 #pragma unroll
-                    for (int ds = 0; ds < G::DS; ds++)
+                    for (int ds = 0; ds < G::DS; ds++) {
                         kreg[ds] = *reinterpret_cast<const s16x8 *>(lds_k + prow * G::PITCH + ds * 32 + g * 8);
-                    int voff = prow * G::PITCH + g * 8;
+                        vreg[ds] = *reinterpret_cast<const s16x8 *>(lds_v + prow * G::PITCH + ds * 32 + g * 8);
+                    }
 #pragma unroll
                     for (int mt = 0; mt < G::MT; mt++) {
                         if (mt < 4) issue(mt);
-                        asm volatile("" : "+v"(voff));  // keep its reads where they are
-                        const short *vrow = lds_v + voff;
                         const int row = tok_row(2 * mt, n >> 3, ocol + (n & 7));
                         const short *qp = lds_q + row * G::PITCH + g * 8;
                         const short *gp = lds_g + row * G::PITCH + g * 8;
@@ -399,8 +435,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
 #pragma unroll
                         for (int ds = 0; ds < G::DS; ds++) {
                             cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32), kreg[ds], cs);
-                            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32),
-                                            *reinterpret_cast<const s16x8 *>(vrow + ds * 32), cp);
+                            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32), vreg[ds], cp);
                         }
                         // queries of accumulator rows g*4 .. g*4+3: halo row 2*mt + g/2,
                         // columns 4*(g%2) .. +3, i.e. four consecutive LDS rows

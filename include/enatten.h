@@ -38,7 +38,7 @@ enum {
 
 /* which kernel family a call is routed to (enatten2d_kernel_path) */
 enum { ENATTEN_PATH_NONE = 0, ENATTEN_PATH_SIMT = 1, ENATTEN_PATH_MFMA = 2,
-       ENATTEN_PATH_MFMA_FUSED = 3 /* enatten_set_path only */ };
+       ENATTEN_PATH_MFMA_FUSED = 3, ENATTEN_PATH_MFMA_SPLIT = 4 /* enatten_set_path only */ };
 
 int enatten_abi_version(void);
 
@@ -54,10 +54,12 @@ int enatten2d_kernel_path(int D, int kernel_size, int dtype);
 
 /*
  * Steer dispatch: 0 = automatic (default), ENATTEN_PATH_SIMT = never use the
- * matrix-core kernels, ENATTEN_PATH_MFMA_FUSED = matrix-core kernels with the
- * fused backward (dQ, dK, dV of the inner tiles from one staging of q, k, v, dO)
- * where it is built (head_dim 128, kernel_size 5, contiguous rows); it reads the
- * inputs once but is not faster than the two-pass backward yet, so it is opt-in.
+ * matrix-core kernels.  The matrix-core backward has two forms: two passes (dQ, then
+ * dK/dV) and one fused kernel that stages q, k, v, dO once (built for head_dim 128,
+ * kernel_size 5, image sides that are multiples of 8, contiguous rows).  Automatic
+ * dispatch takes the fused form where it is built and measured faster (at least 2048
+ * tiles of 8x8 pixels in the call and at least 12 tiles along each image side);
+ * ENATTEN_PATH_MFMA_FUSED takes it wherever it is built, ENATTEN_PATH_MFMA_SPLIT never.
  * Process-wide; meant for tests and tuning.  Returns the previous setting.
  */
 int enatten_set_path(int path);

@@ -22,9 +22,11 @@ def _lib():
     return ensure_built()
 
 
-@pytest.fixture(params=["auto", "simt"])
+@pytest.fixture(params=["auto", "simt", "split"])
 def path(request, _lib):
-    prev = _lib.enatten_set_path(1 if request.param == "simt" else 0)
+    # auto: matrix-core kernels where built (fused or two-pass backward as dispatch
+    # decides); split: matrix-core kernels with the two-pass backward; simt: general kernels
+    prev = _lib.enatten_set_path({"auto": 0, "simt": 1, "split": 4}[request.param])
     yield request.param
     _lib.enatten_set_path(prev)
 
@@ -69,8 +71,8 @@ def test_config2_bf16_readme_shape(side, path):
                                          ((4, 4, 128, 128, 128), BF), ((1, 3, 40, 72, 128), F16),
                                          ((1, 2, 37, 50, 128), BF)])
 def test_fused_backward_path(shape, dtype, _lib):
-    # the opt-in fused backward (dQ, dK, dV of every tile from one staging of q, k, v,
-    # dO) against the oracle: images that are all border, mixed, fp16; the last shape
+    # the fused backward (dQ, dK, dV of every tile from one staging of q, k, v, dO),
+    # forced wherever it is built, against the oracle: images that are all border, mixed, fp16; the last shape
     # has sides that are no multiples of 8 and is served by the two-pass kernels
     from e_natten_amd._lib import PATH_MFMA_FUSED
     prev = _lib.enatten_set_path(PATH_MFMA_FUSED)
