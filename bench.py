@@ -82,66 +82,22 @@ def cpu_baseline(shape, ks, dtype, useful_flop, budget_rows=8):
     }
 
 
-# The benchmark configurations of this operator: (name, B, heads, side, head_dim, k, dtype, q/k scale)
-ALL_CONFIGS = [
-    ("C1 fp32 check", 1, 2, 16, 32, 3, "fp32", 32 ** -0.25),
-    ("C2 README 32", 4, 4, 32, 128, 5, "bf16", 1.0),
-    ("C2 README 64", 4, 4, 64, 128, 5, "bf16", 1.0),
-    ("C2 README 128", 4, 4, 128, 128, 5, "bf16", 1.0),
-    ("C2 README 256", 4, 4, 256, 128, 5, "bf16", 1.0),
-    ("C3 fp32 64", 4, 4, 64, 128, 5, "fp32", 1.0),
-    ("C3 fp32 128", 4, 4, 128, 128, 5, "fp32", 1.0),
-    ("C4 k13", 2, 8, 128, 64, 13, "bf16", 1.0),
-    ("C5 stage1", 8, 2, 112, 32, 7, "bf16", 32 ** -0.25),
-    ("C5 stage2", 8, 4, 56, 32, 7, "bf16", 32 ** -0.25),
-    ("C5 stage3", 8, 8, 28, 32, 7, "bf16", 32 ** -0.25),
-    ("C5 stage4", 8, 16, 14, 32, 7, "bf16", 32 ** -0.25),
-]
-
-
-def run_all_configs():
-    """Kernel times (HIP events around every launch) of every benchmark
-    configuration; prints one JSON line with a list of records."""
-    import torch
-    from e_natten_amd import Natten2d, _lib, kernel_path
-    lib = _lib.load()
-    dev = torch.device("cuda:0")
-    dts = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
-    recs = []
-    for name, B, N, S, D, ks, dt, qk in ALL_CONFIGS:
-        g = torch.Generator().manual_seed(0)
-        q, k, v, d_o = (torch.randn((B, N, S, S, D), generator=g) for _ in range(4))
-        q, k = q * qk, k * qk
-        q, k, v, d_o = (t.to(dts[dt]).to(dev) for t in (q, k, v, d_o))
-        for t in (q, k, v):
-            t.requires_grad_(True)
-        step = lambda: torch.autograd.grad(Natten2d.apply(q, k, v, ks), (q, k, v), d_o)
-        for _ in range(5):
-            step()
-        torch.cuda.synchronize()
-        lib.enatten_profile_enable(1)
-        for _ in range(20):
-            step()
-        torch.cuda.synchronize()
-        lib.enatten_profile_enable(0)
-        us = []
-        for i in range(4):  # forward, dQ pass, dK/dV pass, fused backward (one or the other)
-            n, tot = ctypes.c_int(), ctypes.c_double()
-            lib.enatten_profile_read(i, ctypes.byref(n), ctypes.byref(tot))
-            us.append(tot.value / n.value * 1e3 if n.value else 0.0)
-        qn = B * N * S * S
-        flop = 14.0 * ks * ks * D * qn
-        byt = 11 * qn * D * q.element_size() + 8 * qn
-        tot_us = sum(us)
-        recs.append({"config": name, "shape": [B, N, S, S, D], "k": ks, "dtype": dt,
-                     "path": kernel_path(D, ks, dts[dt]), "fwd_us": us[0], "bwd_dq_us": us[1],
-                     "bwd_dkdv_us": us[2], "bwd_fused_us": us[3], "kernel_us": tot_us,
-                     "useful_tflops": flop / tot_us / 1e6,
-                     "alg_GBps": byt / tot_us / 1e3,
-                     "frac_hbm_peak": byt / tot_us / 1e3 / HBM_PEAK_GBS,
-                     "frac_mfma_peak_useful": flop / tot_us / 1e6 / MFMA_BF16_PEAK_TF})
-        del q, k, v, d_o
-    print(json.dumps({"all_configs": recs}))
+# The benchmark configurations of this operator: name -> (B, heads, side, head_dim, k, dtype);
+# `--config NAME` is a shorthand for the matching --batch/--heads/--side/... flags.
+CONFIGS = {
+    "C1-fp32-check": (1, 2, 16, 32, 3, "fp32"),
+    "C2-README-32": (4, 4, 32, 128, 5, "bf16"),
+    "C2-README-64": (4, 4, 64, 128, 5, "bf16"),
+    "C2-README-128": (4, 4, 128, 128, 5, "bf16"),
+    "C2-README-256": (4, 4, 256, 128, 5, "bf16"),
+    "C3-fp32-64": (4, 4, 64, 128, 5, "fp32"),
+    "C3-fp32-128": (4, 4, 128, 128, 5, "fp32"),
+    "C4-k13": (2, 8, 128, 64, 13, "bf16"),
+    "C5-stage1": (8, 2, 112, 32, 7, "bf16"),
+    "C5-stage2": (8, 4, 56, 32, 7, "bf16"),
+    "C5-stage3": (8, 8, 28, 32, 7, "bf16"),
+    "C5-stage4": (8, 16, 14, 32, 7, "bf16"),
+}
 
 
 def main():
@@ -165,11 +121,12 @@ def main():
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run a plain 256 MiB device copy (calibrates rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
-    ap.add_argument("--all-configs", action="store_true",
-                    help="kernel times of every benchmark configuration instead of the headline run")
+    ap.add_argument("--config", choices=sorted(CONFIGS),
+                    help="one of the named benchmark configurations (sets the shape flags)")
     args = ap.parse_args()
-    if args.all_configs:
-        return run_all_configs()
+    if args.config:
+        (args.batch, args.heads, args.side, args.head_dim, args.kernel_size,
+         args.dtype) = CONFIGS[args.config]
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this operator is measured on one GPU only (--gpus 1); "
                  "it has no cross-GPU path, batch*head slabs are independent")
