@@ -179,6 +179,7 @@ struct Geo {
 // the halos shared by neighbouring tiles meet in the same L2.
 struct Sched {
     int t, t_end, step;
+    int seg_end, skip, hop;  // see make_runs; a strided walk has one endless segment
 };
 __device__ __forceinline__ Sched make_sched(int ntiles, int block, int nblocks) {
     const int xcd = block & 7, slot = block >> 3, slots = nblocks >> 3;
@@ -187,23 +188,40 @@ __device__ __forceinline__ Sched make_sched(int ntiles, int block, int nblocks) 
     sc.t = xcd * per + slot;
     sc.t_end = min(ntiles, (xcd + 1) * per);
     sc.step = slots;
+    sc.seg_end = 0x7fffffff; sc.skip = 0; sc.hop = 0;
     return sc;
 }
 
-// The same split over the XCDs, but every workgroup takes one contiguous run of
-// its XCD's tiles.  With tiles numbered down the columns of an image (tile_of_cm)
-// a workgroup then walks down a column, and consecutive tiles share k-1 of their
-// halo's rows, which stay in LDS.
-__device__ __forceinline__ Sched make_runs(int ntiles, int block, int nblocks) {
+// The same split over the XCDs, but a workgroup takes contiguous segments of its
+// XCD's tiles.  With tiles numbered down the columns of an image (tile_of_cm) a
+// workgroup then walks down a column, and consecutive tiles share k-1 of their
+// halo's rows, which stay in LDS.  `per` tiles go to each XCD, in segments of `seg`
+// tiles; the workgroups of an XCD take segment after segment in turn, so that at
+// any time they are at work on neighbouring columns (or neighbouring parts of one)
+// and the halo columns those share meet in the XCD's L2.  Host side: plan_runs.
+struct Runs {
+    int per, seg;
+};
+__device__ __forceinline__ Sched make_runs(int ntiles, int block, int nblocks, Runs rp) {
     const int xcd = block & 7, slot = block >> 3, slots = nblocks >> 3;
-    const int per = (ntiles + 7) >> 3;
-    const int lo = xcd * per, hi = min(ntiles, lo + per);
-    const int run = (max(hi - lo, 0) + slots - 1) / slots;
+    const int lo = xcd * rp.per;
     Sched sc;
-    sc.t = lo + slot * run;
-    sc.t_end = min(hi, sc.t + run);
+    sc.t = lo + slot * rp.seg;
+    sc.t_end = min(ntiles, lo + rp.per);
     sc.step = 1;
+    sc.seg_end = sc.t + rp.seg;
+    sc.hop = slots * rp.seg;
+    sc.skip = sc.hop - rp.seg;
     return sc;
+}
+// the tile after sc.t (at or beyond sc.t_end: none), and the step to it
+__device__ __forceinline__ int sched_peek(const Sched &sc) {
+    const int tn = sc.t + sc.step;
+    return tn >= sc.seg_end ? tn + sc.skip : tn;
+}
+__device__ __forceinline__ void sched_advance(Sched &sc, int tn) {
+    if (tn >= sc.seg_end) sc.seg_end += sc.hop;
+    sc.t = tn;
 }
 
 struct Tile {
@@ -437,6 +455,33 @@ int persistent_grid(K kernel, int64_t ntiles) {
     const int64_t per_xcd = (ntiles + 7) / 8;
     const int64_t slots = per_xcd < 32 * (int64_t)per_cu ? per_xcd : 32 * (int64_t)per_cu;
     return (int)(8 * slots);
+}
+
+// Segments for make_runs.  While a workgroup's share is at most one column (`colh`
+// tiles) it is one segment.  Several columns in a row would put the workgroups of
+// an XCD on columns that are never neighbours at the same time; then the segments
+// are whole columns, or equal parts of a column, dealt out in turn, chosen for the
+// shortest walk of the busiest workgroup (a segment start costs about half a tile:
+// the whole halo is staged, not 8 rows of it).
+inline Runs plan_runs(int64_t ntiles, int grid, int colh) {
+    const int64_t slots = grid / 8, per = (ntiles + 7) / 8;
+    const int64_t run = (per + slots - 1) / slots;
+    Runs rp{(int)per, (int)run};
+    if (run <= colh) return rp;
+    double best = 1.3 * (2.0 * run + 1.0);  // measured: without the shared L2 lines, 1.3x the time
+    for (int m = 1; m <= 8; m++) {
+        if (colh % m) continue;
+        const int64_t seg = colh / m;
+        const int64_t per_a = (per + seg - 1) / seg * seg;
+        const int64_t rounds = (per_a + slots * seg - 1) / (slots * seg);
+        const double cost = rounds * (2.0 * seg + 1.0);
+        if (cost < best) {
+            best = cost;
+            rp.per = (int)per_a;
+            rp.seg = (int)seg;
+        }
+    }
+    return rp;
 }
 
 }  // namespace

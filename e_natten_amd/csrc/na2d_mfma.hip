@@ -36,13 +36,13 @@ namespace {
 // tiles share in LDS (see make_runs); otherwise a strided walk over row-major tiles
 // with the whole halo staged per tile.
 template <bool BF, int D, int KS, bool ROLL>
-__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles) {
+__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles, Runs rp) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
 
     const Shape &s = a.s;
-    Sched sc = ROLL ? make_runs(ntiles, blockIdx.x, gridDim.x) : make_sched(ntiles, blockIdx.x, gridDim.x);
+    Sched sc = ROLL ? make_runs(ntiles, blockIdx.x, gridDim.x, rp) : make_sched(ntiles, blockIdx.x, gridDim.x);
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS>(lds_k);
     zero_row<D, KS>(lds_v);
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
         for (int ds = 0; ds < G::DS; ds++) qreg[ds] = qnext[ds];
         __syncthreads();
 
-        const int tn = sc.t + sc.step;
+        const int tn = sched_peek(sc);
         const bool more = tn < sc.t_end;
         Tile nxt = cur;
         LaneQ lqn = lq;
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
         __syncthreads();  // every wave is done with this tile's LDS
         cur = nxt;
         lq = lqn;
-        sc.t = tn;
+        sched_advance(sc, tn);
     }
 }
 
@@ -188,14 +188,14 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
 // FRAME: walk only the tiles of the frame of `ts` (the inner tiles are served by
 // the fused backward).
 template <bool BF, int D, int KS, bool FRAME, bool ROLL>
-__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs a, TileSet ts, int ntiles) {
+__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs a, TileSet ts, int ntiles, Runs rp) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
 
     const Shape &s = a.s;
     static_assert(!(FRAME && ROLL), "the frame is not walked by columns");
-    Sched sc = ROLL ? make_runs(ntiles, blockIdx.x, gridDim.x) : make_sched(ntiles, blockIdx.x, gridDim.x);
+    Sched sc = ROLL ? make_runs(ntiles, blockIdx.x, gridDim.x, rp) : make_sched(ntiles, blockIdx.x, gridDim.x);
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS>(lds_k);
     zero_row<D, KS>(lds_v);
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
         const float lse2 = lse_next * kLog2e;
         __syncthreads();
 
-        const int tn = sc.t + sc.step;
+        const int tn = sched_peek(sc);
         const bool more = tn < sc.t_end;
         Tile nxt = cur;
         LaneQ lqn = lq;
@@ -355,7 +355,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
         __syncthreads();
         cur = nxt;
         lq = lqn;
-        sc.t = tn;
+        sched_advance(sc, tn);
     }
 }
 
@@ -399,12 +399,12 @@ __device__ __forceinline__ bool next_block(KeyBlock &b) {
 // queries, a wave's queries are the (4+k-1)^2 halo of its 4x4 keys at a fixed
 // place in it, and the mask depends on the lane only.
 template <bool BF, int D, int KS, bool ROLL>
-__device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, int ntiles,
+__device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, int ntiles, Runs rp,
                                            int block, int nblocks, short *lds_q, short *lds_g,
                                            float2 *lds_stat) {
     using G = Geo<D, KS>;
     const Shape &s = a.s;
-    Sched sc = ROLL ? make_runs(ntiles, block, nblocks) : make_sched(ntiles, block, nblocks);
+    Sched sc = ROLL ? make_runs(ntiles, block, nblocks, rp) : make_sched(ntiles, block, nblocks);
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS>(lds_q);
     zero_row<D, KS>(lds_g);
@@ -497,7 +497,7 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         for (int ds = 0; ds < G::DS; ds++) asm volatile("" : "+v"(kreg[ds]), "+v"(vreg[ds]));
         __syncthreads();
 
-        const int tn = sc.t + sc.step;
+        const int tn = sched_peek(sc);
         const bool more = tn < sc.t_end;
         Tile nxt = cur;
         if (ROLL) rot = (cur.r0 - KS / 2) % G::HR;
@@ -571,7 +571,7 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         load_keys(nxt);
         __syncthreads();
         cur = nxt;
-        sc.t = tn;
+        sched_advance(sc, tn);
     }
 }
 
@@ -760,13 +760,13 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 template <bool BF, int D, int KS, bool ROLL>
 __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArgs a, TileSet ts,
                                                                         int n_inner, int n_frame,
-                                                                        int inner_blocks) {
+                                                                        int inner_blocks, Runs rp) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
     __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
     if ((int)blockIdx.x < inner_blocks)
-        dkdv_inner<BF, D, KS, ROLL>(a, ts, n_inner, blockIdx.x, inner_blocks, lds_q, lds_g, lds_stat);
+        dkdv_inner<BF, D, KS, ROLL>(a, ts, n_inner, rp, blockIdx.x, inner_blocks, lds_q, lds_g, lds_stat);
     else
         dkdv_frame<BF, D, KS>(a, ts, n_frame, blockIdx.x - inner_blocks,
                               gridDim.x - inner_blocks, lds_q, lds_g, lds_stat);
@@ -801,10 +801,10 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
             ProfScope prof(ENATTEN_KERNEL_FWD, "fwd_mfma", st);
             if (roll_pays<D>(nb, grid))
                 hipLaunchKernelGGL((fwd_mfma<BF, D, KS, kRollBuilt<D>>), dim3(grid), dim3(256), 0,
-                                   st, a, tiles_r, tiles_c, (int)nb);
+                                   st, a, tiles_r, tiles_c, (int)nb, plan_runs(nb, grid, tiles_r));
             else
                 hipLaunchKernelGGL((fwd_mfma<BF, D, KS, false>), dim3(grid), dim3(256), 0, st, a,
-                                   tiles_r, tiles_c, (int)nb);
+                                   tiles_r, tiles_c, (int)nb, Runs{0, 0});
         }
         return check_launch("enatten2d_fwd");
     } else {
@@ -831,9 +831,12 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         const int64_t n_inner = slabs * ts.ni_r * ts.ni_c, n_frame = nb - n_inner;
 
         // The fused backward where it is built and measured faster than the two passes:
-        // enough tiles for every CU to walk a while, and images large enough that the
-        // tiles beside the border (1.5x the cost of an inner tile there) are few.
-        const bool fused_pays = nb >= 2048 && tiles_r >= 12 && tiles_c >= 12;
+        // enough tiles for every CU to walk a while, images large enough that the tiles
+        // beside the border (1.5x the cost of an inner tile there) are few, and at most
+        // 48 tiles per workgroup: its workgroups take their tiles in one contiguous run,
+        // so with several columns each they stop meeting their neighbours in L2, while
+        // the two-pass kernels deal columns out in turn (plan_runs) and keep doing so.
+        const bool fused_pays = nb >= 2048 && nb <= 12288 && tiles_r >= 12 && tiles_c >= 12;
         if (path != ENATTEN_PATH_MFMA_SPLIT && fused_bwd_supported(a) &&
             (path == ENATTEN_PATH_MFMA_FUSED || fused_pays)) {
             launch_bwd_fused(a, BF, ts, nb, st);
@@ -845,10 +848,10 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
             if (roll_pays<D>(nb, grid))
                 hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS, false, kRollBuilt<D>>), dim3(grid),
-                                   dim3(256), 0, st, a, ts, (int)nb);
+                                   dim3(256), 0, st, a, ts, (int)nb, plan_runs(nb, grid, tiles_r));
             else
                 hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS, false, false>), dim3(grid), dim3(256), 0,
-                                   st, a, ts, (int)nb);
+                                   st, a, ts, (int)nb, Runs{0, 0});
         }
         {
             // Share the resident workgroups in proportion to the work.  Measured cost
@@ -869,10 +872,11 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
             if (inner_blocks > 0 && roll_pays<D>(n_inner, inner_blocks))
                 hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, kRollBuilt<D>>), dim3(grid), dim3(256),
-                                   0, st, a, ts, (int)n_inner, (int)n_frame, inner_blocks);
+                                   0, st, a, ts, (int)n_inner, (int)n_frame, inner_blocks,
+                                   plan_runs(n_inner, inner_blocks, ts.ni_r));
             else
                 hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, false>), dim3(grid), dim3(256), 0, st,
-                                   a, ts, (int)n_inner, (int)n_frame, inner_blocks);
+                                   a, ts, (int)n_inner, (int)n_frame, inner_blocks, Runs{0, 0});
         }
         return check_launch("enatten2d_bwd");
     } else {

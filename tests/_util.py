@@ -46,15 +46,55 @@ def oracle_all(q, k, v, d_o, ks, scale=1.0, small=False):
     return o, lse, dq, dk, dv
 
 
+def _poison_free_blocks(shape, dtype, dev):
+    """Leave NaN-filled blocks of the operator's output sizes as the only free
+    blocks of torch's caching allocator, so that an output element the kernels
+    fail to write shows up as NaN instead of a stale result of an earlier case."""
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    junk = [torch.full(shape, float("nan"), dtype=dtype, device=dev) for _ in range(4)]
+    junk += [torch.full(shape[:-1], float("nan"), dtype=torch.float32, device=dev) for _ in range(2)]
+    torch.cuda.synchronize()
+    del junk
+
+
 def run_gpu(q, k, v, d_o, ks, scale=1.0):
     """Forward + backward of the HIP operator through autograd on cuda:0."""
     from e_natten_amd import Natten2d
     dev = torch.device("cuda:0")
     qg, kg, vg = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    _poison_free_blocks(tuple(q.shape), q.dtype, dev)
     o = Natten2d.apply(qg, kg, vg, ks, scale)
     o.backward(d_o.to(dev))
     torch.cuda.synchronize()
     return tuple(t.detach().cpu() for t in (o, qg.grad, kg.grad, vg.grad))
+
+
+def run_capi(q, k, v, d_o, ks, scale=1.0):
+    """Forward + backward straight through the C ABI into buffers that hold NaN
+    everywhere beforehand: returns (O, LSE, dQ, dK, dV) on the CPU."""
+    from e_natten_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    code = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}[q.dtype]
+    qd, kd, vd, gd = (t.to(dev).contiguous() for t in (q, k, v, d_o))
+    B, N, H, W, D = q.shape
+    o, dq, dk, dv = (torch.full_like(qd, float("nan")) for _ in range(4))
+    lse = torch.full((B, N, H, W), float("nan"), dtype=torch.float32, device=dev)
+    ws = torch.full((lib.enatten2d_bwd_workspace_bytes(B, N, H, W) // 4 + 1,), float("nan"),
+                    dtype=torch.float32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    rc = lib.enatten2d_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(),
+                           lse.data_ptr(), B, N, H, W, D, ks, code, None, None, None,
+                           float(scale), st)
+    assert rc == 0, _lib.last_error()
+    rc = lib.enatten2d_bwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(),
+                           gd.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                           dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, ks, code, None, None,
+                           None, float(scale), st)
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    return tuple(t.cpu() for t in (o, lse, dq, dk, dv))
 
 
 def assert_close(got, ref, dtype, what):

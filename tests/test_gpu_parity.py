@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from _util import (BF16_REL, FP32_MAX_ABS, O, assert_close, ensure_built, make_inputs,
-                   oracle_all, run_gpu)
+                   oracle_all, run_capi, run_gpu)
 
 pytestmark = pytest.mark.gpu
 
@@ -80,6 +80,29 @@ def test_fused_backward_path(shape, dtype, _lib):
         _case(shape, dtype, 5, what="fused backward %s" % (shape,))
     finally:
         _lib.enatten_set_path(prev)
+
+
+@pytest.mark.parametrize("shape,ks,dtype", [
+    ((8, 16, 16, 64, 128), 5, BF),    # several short columns per workgroup: whole columns in turn
+    ((32, 8, 32, 32, 128), 5, BF),    # the same with taller columns
+    ((4, 10, 128, 128, 128), 5, F16), # quarter columns in turn
+    ((16, 4, 64, 64, 128), 5, BF),    # one column per workgroup
+    ((8, 8, 128, 128, 128), 5, BF),   # two columns per workgroup; fused backward by default
+    ((6, 7, 56, 56, 64), 7, BF),      # row-major walk (head_dim below 128)
+    ((2, 3, 33, 47, 128), 5, BF),     # ragged sides
+    ((2, 2, 24, 40, 48), 5, F32),     # general kernels
+])
+def test_every_output_element_is_written(shape, ks, dtype, path):
+    # The outputs hold NaN before the calls (the kernels must overwrite all of them,
+    # nothing is accumulated); shapes chosen for every way the tiles are dealt to the
+    # workgroups.  Checked against the oracle as well.
+    q, k, v, g = make_inputs(shape, dtype, seed=7)
+    print("case written", shape, dtype, "k=%d" % ks, path, flush=True)
+    o, lse, dq, dk, dv = run_capi(q, k, v, g, ks)
+    assert torch.isfinite(lse).all(), "LSE has elements that were not written"
+    ref = oracle_all(q, k, v, g, ks)
+    assert_close((o, dq, dk, dv), (ref[0], ref[2], ref[3], ref[4]), dtype, "written %s" % (shape,))
+    assert (lse - ref[1]).abs().max().item() <= (1e-4 if dtype == F32 else 2e-2)
 
 
 def test_config2_bf16_side256():
