@@ -132,9 +132,9 @@ def main():
                  "it has no cross-GPU path, batch*head slabs are independent")
 
     import torch
-    from e_natten_amd import Natten2d, _lib, kernel_path
-    if not os.path.exists(_lib.LIB_PATH):
-        from e_natten_amd import build
+    from e_natten_amd import _lib, kernel_path, natten2d
+    from e_natten_amd import build
+    if not (os.path.exists(_lib.LIB_PATH) and os.path.exists(build.TORCH_LIB)):
         build.build()
     lib = _lib.load()
     if args.simt:
@@ -152,7 +152,7 @@ def main():
     q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
 
     def step():
-        o = Natten2d.apply(q, k, v, ks)
+        o = natten2d(q, k, v, ks)
         return torch.autograd.grad(o, (q, k, v), d_o)
 
     for _ in range(args.warmup):
@@ -238,7 +238,7 @@ def main():
                 t.requires_grad_(True)
 
             def step_s():
-                return torch.autograd.grad(Natten2d.apply(qs, ks_, vs, ks), (qs, ks_, vs), gs)
+                return torch.autograd.grad(natten2d(qs, ks_, vs, ks), (qs, ks_, vs), gs)
 
             for _ in range(5):
                 step_s()

@@ -1,4 +1,5 @@
-"""Compile the HIP sources in csrc/ into e_natten_amd/libenatten.so for gfx950.
+"""Compile the HIP sources in csrc/ into e_natten_amd/libenatten.so for gfx950,
+and the native torch binding csrc/torch_shim.cpp into libenatten_torch.so.
 
 Run as ``python -m e_natten_amd.build``.  hipcc cross-compiles without a GPU.
 """
@@ -14,6 +15,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libenatten.so")
+TORCH_LIB = os.path.join(HERE, "libenatten_torch.so")
 SOURCES = ["enatten_capi.hip", "na2d_simt.hip", "na2d_mfma.hip", "na2d_mfma_fused.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -38,8 +40,30 @@ def _compile(src: str) -> str:
     return obj
 
 
+def _build_torch_shim() -> str:
+    """Host-only C++ against the headers of the installed torch; links libenatten.so
+    (found beside it at run time) and the torch libraries the process has loaded."""
+    import torch
+    from torch.utils import cpp_extension
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch.compiled_with_cxx11_abi()),
+           "-I", os.path.join(ROOT, "include")]
+    for inc in cpp_extension.include_paths():
+        cmd += ["-isystem", inc]
+    cmd += ["-isystem", "/opt/rocm/include", os.path.join(CSRC, "torch_shim.cpp"), "-o", TORCH_LIB,
+            "-L", HERE, "-lenatten", "-L", tlib, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch",
+            "-Wl,-rpath,$ORIGIN", "-Wl,--no-as-needed"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building the torch binding failed:\n%s" % r.stderr[-4000:])
+    return TORCH_LIB
+
+
 def build(verbose: bool = False) -> str:
-    """Compile every source and link libenatten.so; returns its path."""
+    """Compile every source and link libenatten.so and the torch binding; returns
+    the path of libenatten.so."""
     os.makedirs(OBJ, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
         objs = list(ex.map(_compile, SOURCES))
@@ -47,8 +71,9 @@ def build(verbose: bool = False) -> str:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s" % r.stderr[-4000:])
+    _build_torch_shim()
     if verbose:
-        print("built", LIB)
+        print("built", LIB, "and", TORCH_LIB)
     return LIB
 
 

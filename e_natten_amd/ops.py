@@ -7,8 +7,18 @@ The device work is done by hand-written HIP kernels for gfx950 reached through
 the C ABI of libenatten.so; the same host shims are also registered as torch
 custom ops ``enatten::na2d_fwd`` / ``enatten::na2d_bwd`` (and ``na1d_*``).  There is no CPU or
 eager fallback: tensors must live on the GPU and the library must be built.
+
+Two host bindings reach the same C ABI.  ``Natten2d`` / ``Natten1d`` are Python
+``autograd.Function``s over ctypes, the mirror of the reference's classes.
+``natten2d`` / ``natten1d`` use the native torch binding (csrc/torch_shim.cpp,
+libenatten_torch.so) when it is built: its forward and backward run no Python,
+which matters because the autograd engine calls a backward on its own thread
+(about a third of the host time per forward+backward on small inputs).  Without
+that library they are ``Natten2d.apply`` / ``Natten1d.apply``.
 """
 from __future__ import annotations
+
+import os
 
 import torch
 
@@ -151,20 +161,38 @@ def _bwd1d_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
     return dq, dk, dv
 
 
-# torch custom ops: thin shims over the C ABI
-_torch_lib = torch.library.Library("enatten", "DEF")
-_torch_lib.define("na2d_fwd(Tensor q, Tensor k, Tensor v, int kernel_size, float scale) "
-                  "-> (Tensor, Tensor)")
-_torch_lib.define("na2d_bwd(Tensor q, Tensor k, Tensor v, Tensor o, Tensor lse, Tensor d_o, "
-                  "int kernel_size, float scale) -> (Tensor, Tensor, Tensor)")
-_torch_lib.impl("na2d_fwd", _fwd_impl, "CompositeExplicitAutograd")
-_torch_lib.impl("na2d_bwd", _bwd_impl, "CompositeExplicitAutograd")
-_torch_lib.define("na1d_fwd(Tensor q, Tensor k, Tensor v, int kernel_size, float scale) "
-                  "-> (Tensor, Tensor)")
-_torch_lib.define("na1d_bwd(Tensor q, Tensor k, Tensor v, Tensor o, Tensor lse, Tensor d_o, "
-                  "int kernel_size, float scale) -> (Tensor, Tensor, Tensor)")
-_torch_lib.impl("na1d_fwd", _fwd1d_impl, "CompositeExplicitAutograd")
-_torch_lib.impl("na1d_bwd", _bwd1d_impl, "CompositeExplicitAutograd")
+def _load_native_binding() -> bool:
+    """Load libenatten_torch.so, which registers the enatten:: operators from C++.
+    It needs libenatten.so beside it; with either file missing the operators are
+    registered from Python below (and fail at the first call if libenatten.so is
+    missing)."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libenatten_torch.so")
+    if os.environ.get("ENATTEN_PYTHON_BINDING") == "1":
+        return False
+    if not (os.path.exists(path) and os.path.exists(_lib.LIB_PATH)):
+        return False
+    _lib.load()
+    torch.ops.load_library(path)
+    return True
+
+
+NATIVE_BINDING = _load_native_binding()
+
+if not NATIVE_BINDING:
+    # torch custom ops: thin shims over the C ABI
+    _torch_lib = torch.library.Library("enatten", "DEF")
+    _torch_lib.define("na2d_fwd(Tensor q, Tensor k, Tensor v, int kernel_size, float scale) "
+                      "-> (Tensor, Tensor)")
+    _torch_lib.define("na2d_bwd(Tensor q, Tensor k, Tensor v, Tensor o, Tensor lse, Tensor d_o, "
+                      "int kernel_size, float scale) -> (Tensor, Tensor, Tensor)")
+    _torch_lib.impl("na2d_fwd", _fwd_impl, "CompositeExplicitAutograd")
+    _torch_lib.impl("na2d_bwd", _bwd_impl, "CompositeExplicitAutograd")
+    _torch_lib.define("na1d_fwd(Tensor q, Tensor k, Tensor v, int kernel_size, float scale) "
+                      "-> (Tensor, Tensor)")
+    _torch_lib.define("na1d_bwd(Tensor q, Tensor k, Tensor v, Tensor o, Tensor lse, Tensor d_o, "
+                      "int kernel_size, float scale) -> (Tensor, Tensor, Tensor)")
+    _torch_lib.impl("na1d_fwd", _fwd1d_impl, "CompositeExplicitAutograd")
+    _torch_lib.impl("na1d_bwd", _bwd1d_impl, "CompositeExplicitAutograd")
 
 
 class Natten2d(torch.autograd.Function):
@@ -194,7 +222,15 @@ class Natten2d(torch.autograd.Function):
         return dQ, dK, dV, None, None
 
 
-natten2d = Natten2d.apply
+def natten2d(q, k, v, kernel_size=7, scale=1.0):
+    """``natten2d(q, k, v, kernel_size) -> out`` on ``[B, heads, H, W, d]`` tensors,
+    differentiable in q, k and v: the reference's entry point
+    (e_natten/triton.py:550, e_natten/__init__.py:1), positional like it."""
+    if not NATIVE_BINDING:
+        return Natten2d.apply(q, k, v, kernel_size, scale)
+    _validate(q, k, v, kernel_size)
+    _require_gpu(q, "natten2d")
+    return torch.ops.enatten.natten2d(q, k, v, kernel_size, float(scale))
 
 
 class Natten1d(torch.autograd.Function):
@@ -217,7 +253,14 @@ class Natten1d(torch.autograd.Function):
         return dQ, dK, dV, None, None
 
 
-natten1d = Natten1d.apply
+def natten1d(q, k, v, kernel_size=7, scale=1.0):
+    """``natten1d(q, k, v, kernel_size) -> out`` on ``[B, heads, T, d]`` tensors
+    (e_natten/triton.py:485, e_natten/__init__.py:1)."""
+    if not NATIVE_BINDING:
+        return Natten1d.apply(q, k, v, kernel_size, scale)
+    _validate(q, k, v, kernel_size, 4)
+    _require_gpu(q, "natten1d")
+    return torch.ops.enatten.natten1d(q, k, v, kernel_size, float(scale))
 
 
 def kernel_path(head_dim: int, kernel_size: int, dtype: torch.dtype) -> str:

@@ -57,7 +57,7 @@ int enatten2d_kernel_path(int D, int kernel_size, int dtype);
  * matrix-core kernels.  The matrix-core backward has two forms: two passes (dQ, then
  * dK/dV) and one fused kernel that stages q, k, v, dO once (built for head_dim 128,
  * kernel_size 5, image sides that are multiples of 8, contiguous rows).  Automatic
- * dispatch takes the fused form where it is built and measured faster (at least 2048
+ * dispatch takes the fused form where it is built and measured faster (2048 to 12288
  * tiles of 8x8 pixels in the call and at least 12 tiles along each image side);
  * ENATTEN_PATH_MFMA_FUSED takes it wherever it is built, ENATTEN_PATH_MFMA_SPLIT never.
  * Process-wide; meant for tests and tuning.  Returns the previous setting.

@@ -20,9 +20,8 @@ BF16_REL = 2e-2       # bfloat16 / float16: max |x - ref| / max |ref|
 
 def ensure_built():
     """Load the HIP library; build it only if no built library is present."""
-    from e_natten_amd import _lib
-    if not os.path.exists(_lib.LIB_PATH):
-        from e_natten_amd import build
+    from e_natten_amd import _lib, build
+    if not (os.path.exists(_lib.LIB_PATH) and os.path.exists(build.TORCH_LIB)):
         build.build()
     return _lib.load()
 
@@ -58,13 +57,15 @@ def _poison_free_blocks(shape, dtype, dev):
     del junk
 
 
-def run_gpu(q, k, v, d_o, ks, scale=1.0):
-    """Forward + backward of the HIP operator through autograd on cuda:0."""
-    from e_natten_amd import Natten2d
+def run_gpu(q, k, v, d_o, ks, scale=1.0, binding="native"):
+    """Forward + backward of the HIP operator through autograd on cuda:0, through
+    `natten2d` (the native torch binding where it is built) or, with
+    binding="python", through the Python autograd.Function."""
+    from e_natten_amd import Natten2d, natten2d
     dev = torch.device("cuda:0")
     qg, kg, vg = (t.to(dev).requires_grad_(True) for t in (q, k, v))
     _poison_free_blocks(tuple(q.shape), q.dtype, dev)
-    o = Natten2d.apply(qg, kg, vg, ks, scale)
+    o = (natten2d if binding == "native" else Natten2d.apply)(qg, kg, vg, ks, scale)
     o.backward(d_o.to(dev))
     torch.cuda.synchronize()
     return tuple(t.detach().cpu() for t in (o, qg.grad, kg.grad, vg.grad))

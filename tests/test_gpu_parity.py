@@ -172,6 +172,47 @@ def test_strided_qkv_views(path):
     assert_close(got, (ref[0], ref[2], ref[3], ref[4]), BF, "strided")
 
 
+def test_native_binding_is_what_runs(_lib):
+    # natten2d goes through the C++ torch binding (no Python in forward or backward);
+    # both bindings give bit-identical results; views, no-grad calls and inputs that
+    # need no gradient behave like any torch operator
+    from e_natten_amd import natten2d, ops
+    assert ops.NATIVE_BINDING, "libenatten_torch.so is not built or failed to load"
+    q, k, v, g = make_inputs((2, 3, 24, 40, 128), BF, 3)
+    a = run_gpu(q, k, v, g, 5, binding="native")
+    b = run_gpu(q, k, v, g, 5, binding="python")
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    qc, kc, vc = (t.cuda() for t in (q, k, v))
+    with torch.no_grad():
+        o = natten2d(qc, kc, vc, 5)
+    assert not o.requires_grad and torch.equal(o.cpu(), a[0])
+    with torch.inference_mode():
+        assert torch.equal(natten2d(qc, kc, vc, 5).cpu(), a[0])
+    kg = kc.clone().requires_grad_(True)
+    o = natten2d(qc, kg, vc, 5)
+    o.backward(g.cuda())
+    assert torch.equal(kg.grad.cpu(), a[2]) and qc.grad is None
+    # strided q, k, v and a non-contiguous upstream gradient
+    B, N, H, W, D, ks = 2, 4, 20, 24, 64, 5
+    gen = torch.Generator().manual_seed(5)
+    qkv = torch.randn(B, H, W, 3, N, D, generator=gen).to(BF)
+    d_o = torch.randn(B, N, H, W, D, generator=gen).to(BF)
+    ref = oracle_all(*(qkv[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3)), d_o, ks, 1.0, small=True)
+    fused = qkv.cuda().requires_grad_(True)
+    qg, kg, vg = (fused[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+    o = natten2d(qg, kg, vg, ks)
+    (o.transpose(2, 3) * d_o.cuda().transpose(2, 3)).sum().backward()
+    grads = fused.grad.cpu()
+    got = (o.detach().cpu(),) + tuple(grads[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+    assert_close(got, (ref[0], ref[2], ref[3], ref[4]), BF, "strided, native binding")
+    # errors keep their classes
+    with pytest.raises(ValueError):
+        torch.ops.enatten.natten2d(qc, kc, vc, 4, 1.0)
+    with pytest.raises(ValueError):
+        torch.ops.enatten.na2d_bwd(qc, kc, vc, qc, torch.empty(1, device="cuda"), qc[:, :1], 5, 1.0)
+
+
 def test_lse_matches_oracle(_lib):
     q, k, v, g = make_inputs((1, 2, 18, 18, 64), BF, 7)
     ref = oracle_all(q, k, v, g, 7, small=True)

@@ -60,6 +60,28 @@ def test_kernel_path_query(lib):
     lib.enatten_set_path(prev)
 
 
+def test_native_torch_binding_registers_operators():
+    # libenatten_torch.so (csrc/torch_shim.cpp) loads without a GPU and registers the
+    # operators from C++; its checks raise the same error classes as the Python side
+    from e_natten_amd import ops
+    assert ops.NATIVE_BINDING, "libenatten_torch.so is not built or failed to load"
+    for name in ("na2d_fwd", "na2d_bwd", "na1d_fwd", "na1d_bwd", "natten2d", "natten1d"):
+        assert hasattr(torch.ops.enatten, name)
+    q = torch.randn(1, 1, 8, 8, 16)
+    with pytest.raises(ValueError, match="odd"):
+        torch.ops.enatten.natten2d(q, q, q, 4, 1.0)
+    with pytest.raises(ValueError, match="smaller"):
+        torch.ops.enatten.natten2d(q, q, q, 9, 1.0)
+    with pytest.raises(ValueError, match="same shape"):
+        torch.ops.enatten.na2d_fwd(q, q[:, :, :4], q, 3, 1.0)
+    with pytest.raises(ValueError, match="dtype"):
+        torch.ops.enatten.natten2d(q.double(), q.double(), q.double(), 3, 1.0)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        torch.ops.enatten.natten2d(q, q, q, 3, 1.0)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        torch.ops.enatten.natten1d(q[0], q[0], q[0], 3, 1.0)
+
+
 def test_python_surface_mirrors_reference():
     import e_natten_amd
     from e_natten_amd import Natten2d, natten2d
