@@ -82,6 +82,27 @@ def test_native_torch_binding_registers_operators():
         torch.ops.enatten.natten1d(q[0], q[0], q[0], 3, 1.0)
 
 
+def test_python_binding_can_be_forced():
+    # ENATTEN_PYTHON_BINDING=1 keeps the native binding out: the operators are then
+    # registered from Python and natten2d is the Python Function's apply
+    import subprocess
+    import sys
+    code = ("import torch, e_natten_amd\n"
+            "from e_natten_amd import ops\n"
+            "assert not ops.NATIVE_BINDING\n"
+            "assert hasattr(torch.ops.enatten, 'na2d_fwd')\n"
+            "q = torch.randn(1, 1, 8, 8, 16)\n"
+            "try:\n"
+            "    e_natten_amd.natten2d(q, q, q, 3)\n"
+            "except RuntimeError as e:\n"
+            "    assert 'no CPU path' in str(e)\n"
+            "else:\n"
+            "    raise SystemExit('CPU tensors were accepted')\n")
+    env = dict(os.environ, ENATTEN_PYTHON_BINDING="1", PYTHONPATH=ROOT)
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+
+
 def test_python_surface_mirrors_reference():
     import e_natten_amd
     from e_natten_amd import Natten2d, natten2d
