@@ -172,7 +172,13 @@ def _load_native_binding() -> bool:
     if not (os.path.exists(path) and os.path.exists(_lib.LIB_PATH)):
         return False
     _lib.load()
-    torch.ops.load_library(path)
+    try:
+        torch.ops.load_library(path)
+    except OSError as e:  # built against another torch: keep working through Python
+        import warnings
+        warnings.warn("e_natten_amd: %s does not load (%s); using the Python binding. Rebuild it "
+                      "with `python -m e_natten_amd.build`." % (path, e), RuntimeWarning)
+        return False
     return True
 
 
