@@ -226,35 +226,42 @@ def main():
         "roofline": roofline,
     }
     if not args.no_sweep:
-        # the other image sides of the reference's benchmark sweep (bench.py:9,34 there),
-        # wall-clock only, a few steps each
-        sweep = []
-        for side in (32, 64, 256):
-            if side == S:
-                continue
-            shp = (B, N, side, side, D)
-            qs, ks_, vs, gs = (torch.randn(shp, generator=g).to(dtype).to(dev) for _ in range(4))
-            for t in (qs, ks_, vs):
-                t.requires_grad_(True)
-
-            def step_s():
-                return torch.autograd.grad(natten2d(qs, ks_, vs, ks), (qs, ks_, vs), gs)
-
+        # The image sides of the reference's benchmark sweeps (bench.py:9 there: forward
+        # only, under no_grad, sides 16..512; bench.py:34: forward+backward, sides
+        # 16..256), wall-clock only, a few steps each.
+        def wall_ms(fn, iters=20):
             for _ in range(5):
-                step_s()
+                fn()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            for _ in range(20):
-                step_s()
+            for _ in range(iters):
+                fn()
             torch.cuda.synchronize()
-            ms = (time.perf_counter() - t0) * 1e3 / 20
+            return (time.perf_counter() - t0) * 1e3 / iters
+
+        sweep = []
+        for side in (16, 32, 64, 128, 256, 512):
+            shp = (B, N, side, side, D)
+            qs, ks_, vs = (torch.randn(shp, generator=g).to(dtype).to(dev) for _ in range(3))
             qn = B * N * side * side
-            fl = 14.0 * ks * ks * D * qn
-            by = 11 * qn * D * qs.element_size() + 8 * qn
-            sweep.append({"side": side, "ms_per_step": ms, "useful_tflops": fl / ms / 1e9,
-                          "path_frac_of_hbm_peak": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                          "mfma_frac_useful": fl / ms / 1e9 / MFMA_BF16_PEAK_TF})
-            del qs, ks_, vs, gs
+            with torch.no_grad():
+                fwd_ms = wall_ms(lambda: natten2d(qs, ks_, vs, ks))
+            rec = {"side": side, "fwd_ms": fwd_ms,
+                   "fwd_frac_of_hbm_peak": (4 * qn * D * qs.element_size() + 4 * qn)
+                   / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            if side <= 256 and side != S:
+                gs = torch.randn(shp, generator=g).to(dtype).to(dev)
+                for t in (qs, ks_, vs):
+                    t.requires_grad_(True)
+                ms = wall_ms(lambda: torch.autograd.grad(natten2d(qs, ks_, vs, ks), (qs, ks_, vs), gs))
+                fl = 14.0 * ks * ks * D * qn
+                by = 11 * qn * D * qs.element_size() + 8 * qn
+                rec.update({"ms_per_step": ms, "useful_tflops": fl / ms / 1e9,
+                            "path_frac_of_hbm_peak": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                            "mfma_frac_useful": fl / ms / 1e9 / MFMA_BF16_PEAK_TF})
+                del gs
+            sweep.append(rec)
+            del qs, ks_, vs
         out["sweep"] = sweep
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(shape, ks, dtype, useful)
