@@ -126,9 +126,14 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
     }
 }
 
-template <int D, int KS>
+template <int D, int KS, int NW = 4>
 struct Geo {
-    static constexpr int TH = 8, TW = 8;          // pixels per workgroup
+    // NW waves own 4x4 pixel blocks, two side by side: a tile of 2*NW x 8 pixels.
+    // Four waves (8x8 pixels) everywhere, except that the forward of a configuration
+    // whose halo leaves room for only one workgroup per CU can use eight (16x8
+    // pixels) where that still fits: two waves per SIMD, and less halo per pixel.
+    static constexpr int TH = 2 * NW, TW = 8;     // pixels per workgroup
+    static constexpr int NT = 64 * NW;            // threads per workgroup
     static constexpr int HR = TH + KS - 1;        // halo of the workgroup tile
     static constexpr int HC = TW + KS - 1;
     static constexpr int SW = 4 + KS - 1;         // halo side of one wave's 4x4 block
@@ -149,13 +154,13 @@ struct Geo {
     static constexpr int DS = D / 32;             // reduction steps over channels
     static constexpr int DT = D / 16;             // 16-channel MFMA row tiles of the output
     static constexpr int NCH = HR * HC * CPR;     // 16-byte chunks per staged halo
-    static constexpr int NL = (NCH + 255) / 256;  // chunks per thread
-    static constexpr int NST = (ROWS + 255) / 256;  // per-query statistics per thread
+    static constexpr int NL = (NCH + NT - 1) / NT;  // chunks per thread
+    static constexpr int NST = (ROWS + NT - 1) / NT;  // per-query statistics per thread
     static constexpr size_t LDS_BYTES =
         (size_t)2 * ROWS * PITCH * sizeof(short) + ROWS * 2 * sizeof(float);
     // waves per SIMD to budget registers for: one per workgroup that LDS admits
     // on a CU (a workgroup puts one wave on each of the four SIMDs), at most 2
-    static constexpr int WAVES = 2 * LDS_BYTES <= 160 * 1024 ? 2 : 1;
+    static constexpr int WAVES = (2 * LDS_BYTES <= 160 * 1024 ? 2 : 1) * (NW / 4);
     // staged LDS row of wave token tk whose halo starts at (orow, ocol) of the
     // staged block; numbers that are no token read the all-zero row
     static __device__ __forceinline__ int token_row(int tk, int orow, int ocol) {
@@ -234,10 +239,10 @@ __device__ __forceinline__ Tile tile_of_cm(int t, int tiles_r, int tiles_c, int 
     tl.bb = t / N; tl.nn = t % N;
     return tl;
 }
-__device__ __forceinline__ Tile tile_of(int t, int tiles_r, int tiles_c, int N) {
+__device__ __forceinline__ Tile tile_of(int t, int tiles_r, int tiles_c, int N, int th = 8) {
     Tile tl;
     tl.c0 = (t % tiles_c) * 8; t /= tiles_c;
-    tl.r0 = (t % tiles_r) * 8; t /= tiles_r;
+    tl.r0 = (t % tiles_r) * th; t /= tiles_r;
     tl.bb = t / N; tl.nn = t % N;
     return tl;
 }
@@ -245,30 +250,30 @@ __device__ __forceinline__ Tile tile_of(int t, int tiles_r, int tiles_c, int N) 
 // Staging plan of one thread: which 16-byte chunks of a halo it moves.  Chunk i of
 // thread t is chunk number t + 256*i of the halo in (row, column, channel-chunk)
 // order.  The plan is the same for every tile, so it is computed once.
-template <int D, int KS>
+template <int D, int KS, int NW = 4>
 struct HaloPlan {
-    int rc[Geo<D, KS>::NL];  // halo row << 8 | halo column of chunk i
+    int rc[Geo<D, KS, NW>::NL];  // halo row << 8 | halo column of chunk i
     int ch8;                 // first channel of the thread's chunks
     int lds0;                // LDS element offset of chunk 0
 };
-template <int D, int KS>
-__device__ __forceinline__ HaloPlan<D, KS> make_plan() {
-    using G = Geo<D, KS>;
-    static_assert(256 % G::CPR == 0, "a thread keeps one channel chunk");
-    HaloPlan<D, KS> pl;
+template <int D, int KS, int NW = 4>
+__device__ __forceinline__ HaloPlan<D, KS, NW> make_plan() {
+    using G = Geo<D, KS, NW>;
+    static_assert(G::NT % G::CPR == 0, "a thread keeps one channel chunk");
+    HaloPlan<D, KS, NW> pl;
     pl.ch8 = (threadIdx.x % G::CPR) * 8;
     pl.lds0 = (threadIdx.x / G::CPR) * G::PITCH + pl.ch8;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
-        int row = threadIdx.x / G::CPR + i * (256 / G::CPR);
+        int row = threadIdx.x / G::CPR + i * (G::NT / G::CPR);
         row = row < G::HR * G::HC ? row : G::HR * G::HC - 1;  // tail: harmless duplicate
         pl.rc[i] = ((row / G::HC) << 8) | (row % G::HC);
     }
     return pl;
 }
-template <int D, int KS>
+template <int D, int KS, int NW = 4>
 struct HaloRegs {
-    u32x4 v[Geo<D, KS>::NL];
+    u32x4 v[Geo<D, KS, NW>::NL];
 };
 // Global -> registers: this thread's share of the halo with origin (hr0, hc0) of
 // one image.  Halo positions at or beyond (rlim, clim) are not needed by any
@@ -276,11 +281,11 @@ struct HaloRegs {
 // stay in bounds and branch-free (the values only ever meet zero probabilities).
 // Addresses are a uniform base plus a 32-bit per-lane byte offset formed with
 // 24-bit multiplies: strides are below 2^22 elements (checked on the host).
-template <int D, int KS>
-__device__ __forceinline__ void halo_fetch(HaloRegs<D, KS> &reg, const HaloPlan<D, KS> &pl,
+template <int D, int KS, int NW = 4>
+__device__ __forceinline__ void halo_fetch(HaloRegs<D, KS, NW> &reg, const HaloPlan<D, KS, NW> &pl,
                                   const short *img, int64_t sh, int64_t sw, int hr0, int hc0,
                                   int rlim, int clim) {
-    using G = Geo<D, KS>;
+    using G = Geo<D, KS, NW>;
     const char *base = reinterpret_cast<const char *>(img + hr0 * sh + hc0 * sw);
     const unsigned sh2 = (unsigned)sh * 2u, sw2 = (unsigned)sw * 2u;
     const int rmax = rlim - 1 - hr0, cmax = clim - 1 - hc0;
@@ -293,26 +298,26 @@ __device__ __forceinline__ void halo_fetch(HaloRegs<D, KS> &reg, const HaloPlan<
     }
 }
 // Registers -> LDS, channel-major with padded pitch.
-template <int D, int KS>
-__device__ __forceinline__ void halo_commit(short *lds, const HaloPlan<D, KS> &pl,
-                                   const HaloRegs<D, KS> &reg) {
-    using G = Geo<D, KS>;
+template <int D, int KS, int NW = 4>
+__device__ __forceinline__ void halo_commit(short *lds, const HaloPlan<D, KS, NW> &pl,
+                                   const HaloRegs<D, KS, NW> &reg) {
+    using G = Geo<D, KS, NW>;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
-        const int row = threadIdx.x / G::CPR + i * (256 / G::CPR);
+        const int row = threadIdx.x / G::CPR + i * (G::NT / G::CPR);
         if (row < G::HR * G::HC)
-            *reinterpret_cast<u32x4 *>(lds + pl.lds0 + i * (256 / G::CPR) * G::PITCH) = reg.v[i];
+            *reinterpret_cast<u32x4 *>(lds + pl.lds0 + i * (G::NT / G::CPR) * G::PITCH) = reg.v[i];
     }
 }
 // Row-range variants for halos whose rows are kept in LDS cyclically (image row y
 // in row slot y % HR): move only the `nrows` image rows from y0 on, all HC columns
 // from hc0 on.  A tile that follows its upper neighbour thus loads only the rows
 // the neighbour's halo did not hold.
-template <int D, int KS>
-__device__ __forceinline__ void halo_fetch_rows(HaloRegs<D, KS> &reg, const HaloPlan<D, KS> &pl,
+template <int D, int KS, int NW = 4>
+__device__ __forceinline__ void halo_fetch_rows(HaloRegs<D, KS, NW> &reg, const HaloPlan<D, KS, NW> &pl,
                                                 const short *img, int64_t sh, int64_t sw, int y0,
                                                 int hc0, int nrows, int rlim, int clim) {
-    using G = Geo<D, KS>;
+    using G = Geo<D, KS, NW>;
     const int yb = min(y0, rlim - 1);
     const char *base = reinterpret_cast<const char *>(img + yb * sh + hc0 * sw);
     const unsigned sh2 = (unsigned)sh * 2u, sw2 = (unsigned)sw * 2u;
@@ -328,14 +333,14 @@ __device__ __forceinline__ void halo_fetch_rows(HaloRegs<D, KS> &reg, const Halo
         }
     }
 }
-template <int D, int KS>
-__device__ __forceinline__ void halo_commit_rows(short *lds, const HaloPlan<D, KS> &pl,
-                                                 const HaloRegs<D, KS> &reg, int y0, int nrows) {
-    using G = Geo<D, KS>;
+template <int D, int KS, int NW = 4>
+__device__ __forceinline__ void halo_commit_rows(short *lds, const HaloPlan<D, KS, NW> &pl,
+                                                 const HaloRegs<D, KS, NW> &reg, int y0, int nrows) {
+    using G = Geo<D, KS, NW>;
     const int rot = y0 % G::HR;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
-        const int pix = threadIdx.x / G::CPR + i * (256 / G::CPR);
+        const int pix = threadIdx.x / G::CPR + i * (G::NT / G::CPR);
         const int r = pl.rc[i] >> 8;
         if (pix < G::HR * G::HC && r < nrows) {
             int slot = rot + r;
@@ -347,9 +352,9 @@ __device__ __forceinline__ void halo_commit_rows(short *lds, const HaloPlan<D, K
 }
 // The spare row stays zero for the whole kernel: padding tokens and tokens
 // outside a wave's halo read it, so they add exact zeros to the second product.
-template <int D, int KS>
+template <int D, int KS, int NW = 4>
 __device__ __forceinline__ void zero_row(short *lds) {
-    using G = Geo<D, KS>;
+    using G = Geo<D, KS, NW>;
     if (threadIdx.x < G::CPR)
         *reinterpret_cast<uint4 *>(lds + G::ZROW * G::PITCH + threadIdx.x * 8) =
             make_uint4(0, 0, 0, 0);
@@ -445,10 +450,10 @@ bool layout_ok(const View &v) {
 // workgroups per CU), never more than there are tiles.  The occupancy of a kernel
 // is queried once.
 template <typename K>
-int persistent_grid(K kernel, int64_t ntiles) {
-    static const int per_cu = [kernel]() {
+int persistent_grid(K kernel, int64_t ntiles, int threads = 256) {
+    static const int per_cu = [kernel, threads]() {
         int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, threads, 0) != hipSuccess || n < 1)
             n = 1;
         return n;
     }();

@@ -35,24 +35,24 @@ namespace {
 // ROLL: walk down the columns of an image and keep the halo rows that consecutive
 // tiles share in LDS (see make_runs); otherwise a strided walk over row-major tiles
 // with the whole halo staged per tile.
-template <bool BF, int D, int KS, bool ROLL>
-__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles, Runs rp) {
-    using G = Geo<D, KS>;
+template <bool BF, int D, int KS, bool ROLL, int NW = 4>
+__global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void fwd_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles, Runs rp) {
+    using G = Geo<D, KS, NW>;
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
 
     const Shape &s = a.s;
     Sched sc = ROLL ? make_runs(ntiles, blockIdx.x, gridDim.x, rp) : make_sched(ntiles, blockIdx.x, gridDim.x);
     if (sc.t >= sc.t_end) return;
-    zero_row<D, KS>(lds_k);
-    zero_row<D, KS>(lds_v);
+    zero_row<D, KS, NW>(lds_k);
+    zero_row<D, KS, NW>(lds_v);
 
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
 
     // registers that carry the next tile while the current one is computed
-    const HaloPlan<D, KS> plan = make_plan<D, KS>();
-    HaloRegs<D, KS> kst, vst;
+    const HaloPlan<D, KS, NW> plan = make_plan<D, KS, NW>();
+    HaloRegs<D, KS, NW> kst, vst;
     s16x8 qnext[G::DS];
     // rows [y0, y0 + nr) of the halo are what LDS does not hold yet
     auto prefetch = [&](const Tile &tl, const LaneQ &lq, int y0, int nr) __attribute__((always_inline)) {
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
     };
 
     auto pick = [&](int t) __attribute__((always_inline)) {
-        return ROLL ? tile_of_cm(t, tiles_r, tiles_c, s.N) : tile_of(t, tiles_r, tiles_c, s.N);
+        return ROLL ? tile_of_cm(t, tiles_r, tiles_c, s.N) : tile_of(t, tiles_r, tiles_c, s.N, G::TH);
     };
     Tile cur = pick(sc.t);
     LaneQ lq = lane_query<KS>(cur, s, wave, n);
@@ -187,9 +187,9 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void fwd_mfma(FwdArgs a, 
 // Per-query math: e_natten/triton.py:383-398.
 // FRAME: walk only the tiles of the frame of `ts` (the inner tiles are served by
 // the fused backward).
-template <bool BF, int D, int KS, bool FRAME, bool ROLL>
-__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs a, TileSet ts, int ntiles, Runs rp) {
-    using G = Geo<D, KS>;
+template <bool BF, int D, int KS, bool FRAME, bool ROLL, int NW = 4>
+__global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void bwd_dq_mfma(BwdArgs a, TileSet ts, int ntiles, Runs rp) {
+    using G = Geo<D, KS, NW>;
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
 
@@ -197,19 +197,19 @@ __global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dq_mfma(BwdArgs 
     static_assert(!(FRAME && ROLL), "the frame is not walked by columns");
     Sched sc = ROLL ? make_runs(ntiles, blockIdx.x, gridDim.x, rp) : make_sched(ntiles, blockIdx.x, gridDim.x);
     if (sc.t >= sc.t_end) return;
-    zero_row<D, KS>(lds_k);
-    zero_row<D, KS>(lds_v);
+    zero_row<D, KS, NW>(lds_k);
+    zero_row<D, KS, NW>(lds_v);
 
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
     auto pick = [&](int t) __attribute__((always_inline)) {
         if constexpr (FRAME) return frame_tile(t, ts, s.N);
         else if constexpr (ROLL) return tile_of_cm(t, ts.tiles_r, ts.tiles_c, s.N);
-        else return tile_of(t, ts.tiles_r, ts.tiles_c, s.N);
+        else return tile_of(t, ts.tiles_r, ts.tiles_c, s.N, G::TH);
     };
 
-    const HaloPlan<D, KS> plan = make_plan<D, KS>();
-    HaloRegs<D, KS> kst, vst;
+    const HaloPlan<D, KS, NW> plan = make_plan<D, KS, NW>();
+    HaloRegs<D, KS, NW> kst, vst;
     s16x8 qnext[G::DS], gnext[G::DS];
     float lse_next = 0.f;
     // rows [y0, y0 + nr) of the halo are what LDS does not hold yet
@@ -790,12 +790,38 @@ bool roll_pays(int64_t ntiles, int grid) {
     return kRollBuilt<D> && ntiles >= (int64_t)4 * grid;
 }
 
+// Eight waves on a 16x8 tile where four on an 8x8 tile would be alone on their CU
+// (their halo leaves LDS for one workgroup) and the taller tile's halo still fits:
+// two waves per SIMD and a fifth to a third less halo per pixel.  Forward and dQ
+// pass at head_dim 64 with kernel_size 11 and 13 (measured: forward 82 -> 55 us at
+// k = 13, 76 -> 53 us at k = 11; dQ pass 92 -> 65 us at k = 11).  At k = 13 the dQ
+// pass does not fit the 256 registers a wave has with two waves per SIMD (it spills
+// and is slower, 95 -> 118 us), so it keeps four waves there.
+template <int D, int KS>
+constexpr bool kTallBuilt =
+    Geo<D, KS, 4>::WAVES == 1 && D <= 64 &&
+    (size_t)2 * Geo<D, KS, 8>::ROWS * Geo<D, KS, 8>::PITCH * sizeof(short) <= 160 * 1024;
+template <int D, int KS>
+constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= 11;
+
 template <bool BF, int D, int KS>
 int fwd_launch(const FwdArgs &a, hipStream_t st) {
     if constexpr (fits<D, KS>()) {
         using G = Geo<D, KS>;
         const int tiles_r = (a.s.H + G::TH - 1) / G::TH, tiles_c = (a.s.W + G::TW - 1) / G::TW;
         const int64_t nb = (int64_t)a.s.B * a.s.N * tiles_r * tiles_c;
+        if constexpr (kTallBuilt<D, KS>) {
+            using G8 = Geo<D, KS, 8>;
+            const int tall_r = (a.s.H + G8::TH - 1) / G8::TH;
+            const int64_t nb8 = (int64_t)a.s.B * a.s.N * tall_r * tiles_c;
+            if (nb8 >= 512) {  // enough tall tiles for every CU to have a few
+                const int grid = persistent_grid(fwd_mfma<BF, D, KS, false, 8>, nb8, G8::NT);
+                ProfScope prof(ENATTEN_KERNEL_FWD, "fwd_mfma", st);
+                hipLaunchKernelGGL((fwd_mfma<BF, D, KS, false, 8>), dim3(grid), dim3(G8::NT), 0, st, a,
+                                   tall_r, tiles_c, (int)nb8, Runs{0, 0});
+                return check_launch("enatten2d_fwd");
+            }
+        }
         const int grid = persistent_grid(fwd_mfma<BF, D, KS, false>, nb);
         {
             ProfScope prof(ENATTEN_KERNEL_FWD, "fwd_mfma", st);
@@ -843,7 +869,21 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             return check_launch("enatten2d_bwd");
         }
 
-        {
+        bool dq_done = false;
+        if constexpr (kTallDqBuilt<D, KS>) {
+            using G8 = Geo<D, KS, 8>;
+            TileSet tall = ts;  // only the tile counts are used by this pass
+            tall.tiles_r = (a.s.H + G8::TH - 1) / G8::TH;
+            const int64_t nb8 = slabs * tall.tiles_r * tiles_c;
+            if (nb8 >= 512) {
+                const int grid = persistent_grid(bwd_dq_mfma<BF, D, KS, false, false, 8>, nb8, G8::NT);
+                ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
+                hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS, false, false, 8>), dim3(grid), dim3(G8::NT),
+                                   0, st, a, tall, (int)nb8, Runs{0, 0});
+                dq_done = true;
+            }
+        }
+        if (!dq_done) {
             const int grid = persistent_grid(bwd_dq_mfma<BF, D, KS, false, false>, nb);
             ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
             if (roll_pays<D>(nb, grid))

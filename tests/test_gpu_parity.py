@@ -89,6 +89,8 @@ def test_fused_backward_path(shape, dtype, _lib):
     ((16, 4, 64, 64, 128), 5, BF),    # one column per workgroup
     ((8, 8, 128, 128, 128), 5, BF),   # two columns per workgroup; fused backward by default
     ((6, 7, 56, 56, 64), 7, BF),      # row-major walk (head_dim below 128)
+    ((8, 8, 72, 40, 64), 13, BF),     # 16x8 tiles of eight waves (forward), ragged last tile row
+    ((4, 8, 56, 88, 64), 11, F16),    # 16x8 tiles in the forward and the dQ pass
     ((2, 3, 33, 47, 128), 5, BF),     # ragged sides
     ((2, 2, 24, 40, 48), 5, F32),     # general kernels
 ])
