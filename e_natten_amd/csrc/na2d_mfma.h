@@ -448,12 +448,13 @@ bool layout_ok(const View &v) {
 
 // Persistent grid: as many workgroups as stay resident at once (8 XCDs x 32 CUs x
 // workgroups per CU), never more than there are tiles.  The occupancy of a kernel
-// is queried once.
-template <typename K>
-int persistent_grid(K kernel, int64_t ntiles, int threads = 256) {
-    static const int per_cu = [kernel, threads]() {
+// is queried once; the kernel is a template argument so that every instantiation
+// has its own cached value (kernels of one signature share a function type).
+template <auto KERNEL>
+int persistent_grid(int64_t ntiles, int threads = 256) {
+    static const int per_cu = [threads]() {
         int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, threads, 0) != hipSuccess || n < 1)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, KERNEL, threads, 0) != hipSuccess || n < 1)
             n = 1;
         return n;
     }();

@@ -815,14 +815,14 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
             const int tall_r = (a.s.H + G8::TH - 1) / G8::TH;
             const int64_t nb8 = (int64_t)a.s.B * a.s.N * tall_r * tiles_c;
             if (nb8 >= 512) {  // enough tall tiles for every CU to have a few
-                const int grid = persistent_grid(fwd_mfma<BF, D, KS, false, 8>, nb8, G8::NT);
+                const int grid = persistent_grid<fwd_mfma<BF, D, KS, false, 8>>(nb8, G8::NT);
                 ProfScope prof(ENATTEN_KERNEL_FWD, "fwd_mfma", st);
                 hipLaunchKernelGGL((fwd_mfma<BF, D, KS, false, 8>), dim3(grid), dim3(G8::NT), 0, st, a,
                                    tall_r, tiles_c, (int)nb8, Runs{0, 0});
                 return check_launch("enatten2d_fwd");
             }
         }
-        const int grid = persistent_grid(fwd_mfma<BF, D, KS, false>, nb);
+        const int grid = persistent_grid<fwd_mfma<BF, D, KS, false>>(nb);
         {
             ProfScope prof(ENATTEN_KERNEL_FWD, "fwd_mfma", st);
             if (roll_pays<D>(nb, grid))
@@ -876,7 +876,7 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             tall.tiles_r = (a.s.H + G8::TH - 1) / G8::TH;
             const int64_t nb8 = slabs * tall.tiles_r * tiles_c;
             if (nb8 >= 512) {
-                const int grid = persistent_grid(bwd_dq_mfma<BF, D, KS, false, false, 8>, nb8, G8::NT);
+                const int grid = persistent_grid<bwd_dq_mfma<BF, D, KS, false, false, 8>>(nb8, G8::NT);
                 ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
                 hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS, false, false, 8>), dim3(grid), dim3(G8::NT),
                                    0, st, a, tall, (int)nb8, Runs{0, 0});
@@ -884,7 +884,7 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             }
         }
         if (!dq_done) {
-            const int grid = persistent_grid(bwd_dq_mfma<BF, D, KS, false, false>, nb);
+            const int grid = persistent_grid<bwd_dq_mfma<BF, D, KS, false, false>>(nb);
             ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
             if (roll_pays<D>(nb, grid))
                 hipLaunchKernelGGL((bwd_dq_mfma<BF, D, KS, false, kRollBuilt<D>>), dim3(grid),
@@ -898,7 +898,7 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             // of a frame tile in inner tiles: about 2 when the inner tiles are bound
             // by arithmetic (d <= 64), about 1.15 when they are bound by HBM (d = 128).
             const double cost = D >= 128 ? 1.15 : 2.0;
-            const int grid = persistent_grid(bwd_dkdv_mfma<BF, D, KS, false>, nb);
+            const int grid = persistent_grid<bwd_dkdv_mfma<BF, D, KS, false>>(nb);
             int inner_blocks = 0;
             if (n_frame == 0) {
                 inner_blocks = grid;
