@@ -160,7 +160,7 @@ struct Geo {
         (size_t)2 * ROWS * PITCH * sizeof(short) + ROWS * 2 * sizeof(float);
     // waves per SIMD to budget registers for: one per workgroup that LDS admits
     // on a CU (a workgroup puts one wave on each of the four SIMDs), at most 2
-    static constexpr int WAVES = (2 * LDS_BYTES <= 160 * 1024 ? 2 : 1) * (NW / 4);
+    static constexpr int WAVES = NW == 4 ? (2 * LDS_BYTES <= 160 * 1024 ? 2 : 1) : 2;
     // staged LDS row of wave token tk whose halo starts at (orow, ocol) of the
     // staged block; numbers that are no token read the all-zero row
     static __device__ __forceinline__ int token_row(int tk, int orow, int ocol) {

@@ -790,16 +790,17 @@ bool roll_pays(int64_t ntiles, int grid) {
     return kRollBuilt<D> && ntiles >= (int64_t)4 * grid;
 }
 
-// Eight waves on a 16x8 tile where four on an 8x8 tile would be alone on their CU
-// (their halo leaves LDS for one workgroup) and the taller tile's halo still fits:
-// two waves per SIMD and a fifth to a third less halo per pixel.  Forward and dQ
-// pass at head_dim 64 with kernel_size 11 and 13 (measured: forward 82 -> 55 us at
-// k = 13, 76 -> 53 us at k = 11; dQ pass 92 -> 65 us at k = 11).  At k = 13 the dQ
-// pass does not fit the 256 registers a wave has with two waves per SIMD (it spills
-// and is slower, 95 -> 118 us), so it keeps four waves there.
+// Eight waves on a 16x8 tile instead of four on an 8x8 tile, for head_dim 64 with
+// kernel_size >= 7 where the taller tile's halo fits LDS: a fifth to a third less halo
+// per pixel, and at k = 11 and 13, where the halo of an 8x8 tile leaves LDS for one
+// workgroup per CU, two waves per SIMD instead of one.  Measured at B4 N4 128x128
+// (8x8 -> 16x8, us): forward 40 -> 39 (k=7), 76 -> 53 (k=11), 82 -> 55 (k=13); dQ pass
+// 59 -> 48 (k=7), 82 -> 59 (k=9), 92 -> 65 (k=11).  Not used where it was measured
+// slower or no faster: k <= 5, head_dim 32, and the dQ pass at k = 13, which does not
+// fit the 256 registers a wave has at two waves per SIMD (it spills: 95 -> 118 us).
 template <int D, int KS>
 constexpr bool kTallBuilt =
-    Geo<D, KS, 4>::WAVES == 1 && D <= 64 &&
+    D == 64 && KS >= 7 &&
     (size_t)2 * Geo<D, KS, 8>::ROWS * Geo<D, KS, 8>::PITCH * sizeof(short) <= 160 * 1024;
 template <int D, int KS>
 constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= 11;
