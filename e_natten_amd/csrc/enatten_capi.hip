@@ -37,9 +37,9 @@ constexpr int kProfMax = 8192;
 
 ProfScope::ProfScope(int kernel_slot, const char *kernel_name, hipStream_t stream)
     : slot(kernel_slot), st(stream), rec(nullptr) {
-    g_prof[slot].name = kernel_name;
-    if (!g_prof_on) return;
+    if (!g_prof_on) return;  // nothing is written while timing is off: launches stay re-entrant
     ProfSlot &ps = g_prof[slot];
+    ps.name = kernel_name;
     if (ps.calls++ % g_prof_period != 0) return;
     if (ps.used >= kProfMax) return;
     if (ps.used == (int)ps.recs.size()) {
