@@ -59,7 +59,7 @@ def cpu_baseline(shape, ks, dtype, useful_flop, budget_rows=8):
     r1 = min(H, r0 + budget_rows)
     qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
     t0 = time.perf_counter()
-    o = O.natten2d_loops(qq, kk, vv, ks, False, (r0, r1))
+    o = O.natten2d_loops(qq, kk, vv, ks, (r0, r1))
     o.backward(d_o)
     loops_s = (time.perf_counter() - t0) * H / (r1 - r0)
 

@@ -25,13 +25,12 @@ Pinning status (see tests/test_oracle_*.py):
   forward O, LSE             dense-mask SDPA, brute force, k=1, k=H=W, shifts
   dQ, dK, dV                 fp64 autograd of two independent forwards,
                              torch.autograd.gradcheck, sum invariants
-  Natten2dLoops(clean)       equals the gather oracle
-  Natten2dLoops(reference_quirks=True)   parity unpinned: it predicts two
-                             accidental behaviours of e_natten/pytorch.py (dQ
-                             only for the first tile, a shifted window for a
-                             few rows when k//2 is not a multiple of 3); the
-                             reference was read, not run, so the prediction is
-                             not checked against it.
+  Natten2dLoops              equals the gather oracle
+Every function here is pinned by one of those checks.  Two accidental behaviours
+of e_natten/pytorch.py are deliberately NOT restated (they contradict its own
+backward, the Triton kernels and the NATTEN definition): its tile offset rule
+(:25-31) shifts the window of a few rows when k//2 is not a multiple of 3, and
+its dQ loop (:230-231) only visits the first tile.
 """
 from __future__ import annotations
 
@@ -257,20 +256,6 @@ def natten2d_brute(q, k, v, kernel_size: int, scale: float = 1.0):
 REF_TILE = 3  # e_natten/pytorch.py:5
 
 
-def _quirky_tile_offset(origin: int, j: int, L: int, slab_start: int, k: int) -> int:
-    """Offset rule of e_natten/pytorch.py:25-31 as written there.
-
-    It returns ``j`` for interior queries even when the tile's key slab was
-    clamped to the image edge, which is off by one or two rows whenever k//2
-    is not a multiple of the tile size 3 (k = 3 and k = 9).
-    """
-    if origin + j <= k // 2:
-        return 0
-    if origin + j >= L - k // 2 - 1:
-        return L - slab_start - k
-    return j
-
-
 def _softmax_jvp(p: torch.Tensor, dp: torch.Tensor) -> torch.Tensor:
     """(diag(p) - p p^T) dp over the last axis: what the reference builds as a
     dense Jacobian (e_natten/pytorch.py:33-43) and multiplies by dP (:256)."""
@@ -288,17 +273,15 @@ class Natten2dLoops(torch.autograd.Function):
                key by walking the inverse neighbourhood and recomputing each
                contributing query's softmax (:261-288).
 
-    ``reference_quirks=False`` (default) gives the intended operator: the
-    in-slab offset is ``win_start(query) - slab_start`` and dQ is produced for
-    every tile (the loop the reference has commented out at :228-229).
-    ``reference_quirks=True`` keeps the file's literal behaviour (offset rule
-    of :25-31, dQ for the first tile only, :230-231).
+    The in-slab offset is ``win_start(query) - slab_start`` (the file's own rule,
+    :25-31, is wrong for k = 3 and 9) and dQ is produced for every tile (the loop
+    the reference has commented out at :228-229).
     ``rows=(r0, r1)`` restricts the outer row loops to that band so a bounded
     sample of the work can be timed; outputs outside the band stay zero.
     """
 
     @staticmethod
-    def forward(ctx, q, k, v, kernel_size=7, reference_quirks=False, rows=None):
+    def forward(ctx, q, k, v, kernel_size=7, rows=None):
         _check(q, k, v, kernel_size)
         B, N, H, W, D = q.shape
         ks = kernel_size
@@ -315,25 +298,21 @@ class Natten2dLoops(torch.autograd.Function):
                     if not (r0 <= tx + ix < r1):
                         continue
                     for iy in range(min(REF_TILE, W - ty)):
-                        if reference_quirks:
-                            ox = _quirky_tile_offset(tx, ix, H, sx0, ks)
-                            oy = _quirky_tile_offset(ty, iy, W, sy0, ks)
-                        else:
-                            ox = win_start(tx + ix, H, ks) - sx0
-                            oy = win_start(ty + iy, W, ks) - sy0
+                        ox = win_start(tx + ix, H, ks) - sx0
+                        oy = win_start(ty + iy, W, ks) - sy0
                         kw = k_slab[:, :, ox:ox + ks, oy:oy + ks].reshape(B, N, ks * ks, D)
                         vw = v_slab[:, :, ox:ox + ks, oy:oy + ks].reshape(B, N, ks * ks, D)
                         qv = q[:, :, tx + ix, ty + iy]  # [B, N, D]
                         p = torch.softmax(torch.einsum("bnd,bnjd->bnj", qv, kw), dim=-1)
                         out[:, :, tx + ix, ty + iy] = torch.einsum("bnj,bnjd->bnd", p, vw)
         ctx.save_for_backward(q, k, v)
-        ctx.ks, ctx.quirks, ctx.rows = ks, reference_quirks, (r0, r1)
+        ctx.ks, ctx.rows = ks, (r0, r1)
         return out
 
     @staticmethod
     def backward(ctx, d_o):
         q, k, v = ctx.saved_tensors
-        ks, quirks, (r0, r1) = ctx.ks, ctx.quirks, ctx.rows
+        ks, (r0, r1) = ctx.ks, ctx.rows
         B, N, H, W, D = q.shape
         slab = REF_TILE + ks - 1
         dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
@@ -346,22 +325,14 @@ class Natten2dLoops(torch.autograd.Function):
             return p, _softmax_jvp(p, dp), kw
 
         # dQ, tile by tile
-        tiles_x = [0] if quirks else range(r0 - r0 % REF_TILE, r1, REF_TILE)
-        tiles_y = [0] if quirks else range(0, W, REF_TILE)
-        for tx in tiles_x:
-            sx0 = win_start(tx, H, ks)
-            for ty in tiles_y:
-                sy0 = win_start(ty, W, ks)
+        for tx in range(r0 - r0 % REF_TILE, r1, REF_TILE):
+            for ty in range(0, W, REF_TILE):
                 for ix in range(min(REF_TILE, H - tx)):
-                    if not quirks and not (r0 <= tx + ix < r1):
+                    if not (r0 <= tx + ix < r1):
                         continue
                     for iy in range(min(REF_TILE, W - ty)):
-                        if quirks:
-                            x0 = sx0 + _quirky_tile_offset(tx, ix, H, sx0, ks)
-                            y0 = sy0 + _quirky_tile_offset(ty, iy, W, sy0, ks)
-                        else:
-                            x0 = win_start(tx + ix, H, ks)
-                            y0 = win_start(ty + iy, W, ks)
+                        x0 = win_start(tx + ix, H, ks)
+                        y0 = win_start(ty + iy, W, ks)
                         _, ds, kw = query_terms(tx + ix, ty + iy, x0, y0)
                         dq[:, :, tx + ix, ty + iy] = torch.einsum("bnj,bnjd->bnd", ds, kw)
 
@@ -378,11 +349,11 @@ class Natten2dLoops(torch.autograd.Function):
                         slot = (x - wx) * ks + (y - wy)
                         dk[:, :, x, y] += q[:, :, xi, yi] * ds[:, :, slot, None]
                         dv[:, :, x, y] += d_o[:, :, xi, yi] * p[:, :, slot, None]
-        return dq, dk, dv, None, None, None
+        return dq, dk, dv, None, None
 
 
-def natten2d_loops(q, k, v, kernel_size=7, reference_quirks=False, rows=None):
-    return Natten2dLoops.apply(q, k, v, kernel_size, reference_quirks, rows)
+def natten2d_loops(q, k, v, kernel_size=7, rows=None):
+    return Natten2dLoops.apply(q, k, v, kernel_size, rows)
 
 
 # --------------------------------------------------------------------------

@@ -68,15 +68,6 @@ def test_loop_restatement_backward_equals_explicit():
         assert O.max_abs_err(rv, dv) < 1e-11
 
 
-def test_loop_restatement_quirks_dq_first_tile_only():
-    q, kk, v, g = _rand((1, 1, 8, 8, 3), 5)
-    rq, rk, rv = _autograd(lambda a, b, c: O.natten2d_loops(a, b, c, 5, True), q, kk, v, g)
-    _, _, dq, dk, dv = O.natten2d_explicit(q, kk, v, g, 5)
-    assert O.max_abs_err(rq[:, :, :3, :3], dq[:, :, :3, :3]) < 1e-11
-    assert rq[:, :, 3:].abs().max() == 0 and rq[:, :, :, 3:].abs().max() == 0
-    assert O.max_abs_err(rk, dk) < 1e-11 and O.max_abs_err(rv, dv) < 1e-11
-
-
 @pytest.mark.parametrize("shape,k,scale", [((2, 3, 16, 16, 2), 3, 1.0), ((1, 2, 14, 14, 32), 7, 32 ** -0.5),
                                            ((1, 1, 20, 17, 8), 13, 1.0), ((1, 2, 16, 16, 2), 11, 1.0)])
 def test_c_oracle_backward(shape, k, scale, c_oracle):

@@ -82,24 +82,9 @@ def test_loop_restatement_clean_equals_gather(k):
 def test_loop_restatement_row_band():
     q, kk, v = _rand((1, 1, 12, 9, 4), 8)
     o = O.natten2d_gather(q, kk, v, 5)
-    ol = O.natten2d_loops(q, kk, v, 5, False, (4, 8))
+    ol = O.natten2d_loops(q, kk, v, 5, (4, 8))
     assert O.max_abs_err(o[:, :, 4:8], ol[:, :, 4:8]) < 1e-12
     assert ol[:, :, :4].abs().max() == 0 and ol[:, :, 8:].abs().max() == 0
-
-
-def test_loop_restatement_quirks_mode_differs_only_where_predicted():
-    # k=5: k//2 = 2 ... the literal offset rule is exact for k in {5, 7, 11, 13}
-    q, kk, v = _rand((1, 1, 16, 16, 4), 9)
-    o = O.natten2d_gather(q, kk, v, 5)
-    assert O.max_abs_err(O.natten2d_loops(q, kk, v, 5, True), o) < 1e-12
-    # k=3: rows/cols with index 2 pick a window shifted by one
-    o3 = O.natten2d_gather(q, kk, v, 3)
-    ol3 = O.natten2d_loops(q, kk, v, 3, True)
-    bad = (o3 - ol3).abs().amax(dim=(0, 1, 4)) > 1e-9
-    expect = torch.zeros(16, 16, dtype=torch.bool)
-    expect[2, :] = True
-    expect[:, 2] = True
-    assert torch.equal(bad, expect)
 
 
 @pytest.mark.parametrize("shape,k", [((2, 3, 16, 16, 2), 3), ((1, 2, 14, 14, 32), 7), ((1, 1, 20, 17, 8), 13)])
