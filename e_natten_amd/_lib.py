@@ -8,6 +8,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libenatten.so")
 
+ABI_VERSION = 2  # ENATTEN_ABI_VERSION of include/enatten.h
 F32, BF16, F16 = 0, 1, 2
 PATH_NONE, PATH_SIMT, PATH_MFMA, PATH_MFMA_FUSED, PATH_MFMA_SPLIT = 0, 1, 2, 3, 4
 
@@ -24,12 +25,12 @@ SIGNATURES = {
     "enatten_last_error": (ctypes.c_char_p, []),
     "enatten2d_kernel_path": (_i, [_i, _i, _i]),
     "enatten_set_path": (_i, [_i]),
-    "enatten2d_fwd": (_i, [_vp] * 5 + [_i] * 7 + [_sp] * 3 + [ctypes.c_float, _vp]),
+    "enatten2d_fwd": (_i, [_vp] * 5 + [_i] * 7 + [_sp] * 4 + [ctypes.c_float, _vp]),
     "enatten2d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 4),
-    "enatten2d_bwd": (_i, [_vp] * 10 + [_i] * 7 + [_sp] * 3 + [ctypes.c_float, _vp]),
-    "enatten1d_fwd": (_i, [_vp] * 5 + [_i] * 6 + [_sp] * 3 + [ctypes.c_float, _vp]),
+    "enatten2d_bwd": (_i, [_vp] * 10 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
+    "enatten1d_fwd": (_i, [_vp] * 5 + [_i] * 6 + [_sp] * 4 + [ctypes.c_float, _vp]),
     "enatten1d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 3),
-    "enatten1d_bwd": (_i, [_vp] * 10 + [_i] * 6 + [_sp] * 3 + [ctypes.c_float, _vp]),
+    "enatten1d_bwd": (_i, [_vp] * 10 + [_i] * 6 + [_sp] * 5 + [ctypes.c_float, _vp]),
     "enatten_profile_enable": (_i, [_i]),
     "enatten_profile_read": (_i, [_i, ctypes.POINTER(_i), ctypes.POINTER(ctypes.c_double)]),
     "enatten_profile_kernel_name": (ctypes.c_char_p, [_i]),
@@ -51,7 +52,7 @@ def load() -> ctypes.CDLL:
             for name, (res, args) in SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.restype, fn.argtypes = res, args
-            if lib.enatten_abi_version() != 1:
+            if lib.enatten_abi_version() != ABI_VERSION:
                 raise ImportError("libenatten.so has an unexpected ABI version")
             _lib = lib
     return _lib

@@ -4,7 +4,6 @@
 #include <stdio.h>
 
 #include <atomic>
-#include <vector>
 
 #include "na2d_common.h"
 
@@ -18,44 +17,6 @@ void set_error(const char *fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
-}
-
-// ---- optional per-kernel event timing -------------------------------------
-namespace {
-struct ProfRec { hipEvent_t e0, e1; };
-struct ProfSlot {
-    std::vector<ProfRec> recs;  // events are created once and reused
-    int used = 0;
-    int calls = 0;
-    const char *name = "";
-};
-ProfSlot g_prof[ENATTEN_KERNEL_COUNT];
-bool g_prof_on = false;
-int g_prof_period = 1;  // every g_prof_period-th launch of a kernel is timed
-constexpr int kProfMax = 8192;
-}  // namespace
-
-ProfScope::ProfScope(int kernel_slot, const char *kernel_name, hipStream_t stream)
-    : slot(kernel_slot), st(stream), rec(nullptr) {
-    if (!g_prof_on) return;  // nothing is written while timing is off: launches stay re-entrant
-    ProfSlot &ps = g_prof[slot];
-    ps.name = kernel_name;
-    if (ps.calls++ % g_prof_period != 0) return;
-    if (ps.used >= kProfMax) return;
-    if (ps.used == (int)ps.recs.size()) {
-        ProfRec r;
-        if (hipEventCreate(&r.e0) != hipSuccess || hipEventCreate(&r.e1) != hipSuccess) return;
-        ps.recs.push_back(r);
-    }
-    ProfRec *r = &ps.recs[ps.used];
-    if (hipEventRecord(r->e0, st) != hipSuccess) return;
-    rec = r;
-}
-
-ProfScope::~ProfScope() {
-    if (!rec) return;
-    ProfRec *r = static_cast<ProfRec *>(rec);
-    if (hipEventRecord(r->e1, st) == hipSuccess) g_prof[slot].used++;
 }
 
 namespace {
@@ -87,9 +48,15 @@ int check_shape(const char *fn, int B, int N, int H, int W, int D, int ks, int d
         set_error("%s: image %dx%d is smaller than kernel_size %d", fn, H, W, ks);
         return ENATTEN_EINVAL;
     }
-    if ((int64_t)B * N * H * W * D >= ((int64_t)1 << 40)) {
-        set_error("%s: tensor too large", fn);
-        return ENATTEN_EUNSUPPORTED;
+    // elements of one tensor, checked factor by factor so that nothing overflows
+    const int64_t limit = (int64_t)1 << 40;
+    int64_t count = 1;
+    for (const int f : {B, N, H, W, D}) {
+        if (count > limit / f) {
+            set_error("%s: tensor too large (more than 2^40 elements)", fn);
+            return ENATTEN_EUNSUPPORTED;
+        }
+        count *= f;
     }
     return ENATTEN_OK;
 }
@@ -148,7 +115,7 @@ int enatten_set_path(int path) {
 int enatten2d_fwd(const void *q, const void *k, const void *v, void *o, float *lse, int B,
                   int heads, int H, int W, int D, int kernel_size, int dtype,
                   const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
-                  float scale, void *stream) {
+                  const int64_t *o_strides, float scale, void *stream) {
     const char *fn = "enatten2d_fwd";
     int rc = check_shape(fn, B, heads, H, W, D, kernel_size, dtype);
     if (rc) return rc;
@@ -156,11 +123,7 @@ int enatten2d_fwd(const void *q, const void *k, const void *v, void *o, float *l
     if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
     if ((rc = make_view(fn, "k", k, k_strides, heads, H, W, D, &a.k))) return rc;
     if ((rc = make_view(fn, "v", v, v_strides, heads, H, W, D, &a.v))) return rc;
-    if (!o) {
-        set_error("%s: o is NULL", fn);
-        return ENATTEN_EINVAL;
-    }
-    a.o = o;
+    if ((rc = make_view(fn, "o", o, o_strides, heads, H, W, D, &a.o))) return rc;
     a.lse = lse;
     a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -177,7 +140,8 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o, co
                   const float *lse, void *dq, void *dk, void *dv, void *workspace, int B,
                   int heads, int H, int W, int D, int kernel_size, int dtype,
                   const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
-                  float scale, void *stream) {
+                  const int64_t *o_strides, const int64_t *do_strides, float scale,
+                  void *stream) {
     const char *fn = "enatten2d_bwd";
     int rc = check_shape(fn, B, heads, H, W, D, kernel_size, dtype);
     if (rc) return rc;
@@ -185,11 +149,13 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o, co
     if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
     if ((rc = make_view(fn, "k", k, k_strides, heads, H, W, D, &a.k))) return rc;
     if ((rc = make_view(fn, "v", v, v_strides, heads, H, W, D, &a.v))) return rc;
-    if (!o || !d_o || !lse || !dq || !dk || !dv || !workspace) {
-        set_error("%s: o, d_o, lse, dq, dk, dv and workspace must all be non-NULL", fn);
+    if ((rc = make_view(fn, "o", o, o_strides, heads, H, W, D, &a.o))) return rc;
+    if ((rc = make_view(fn, "d_o", d_o, do_strides, heads, H, W, D, &a.d_o))) return rc;
+    if (!lse || !dq || !dk || !dv || !workspace) {
+        set_error("%s: lse, dq, dk, dv and workspace must all be non-NULL", fn);
         return ENATTEN_EINVAL;
     }
-    a.o = o; a.d_o = d_o; a.lse = lse;
+    a.lse = lse;
     a.dq = dq; a.dk = dk; a.dv = dv;
     a.delta = static_cast<float *>(workspace);
     a.zinv = a.delta + (size_t)B * heads * H * W;
@@ -221,18 +187,21 @@ static int view_1d(const char *fn, const char *name, const void *p, const int64_
     return ENATTEN_OK;
 }
 
+// A sequence is a 1 x T image with a 1 x k window: the size limit applies to
+// B * heads * T * D elements.
 static int check_shape_1d(const char *fn, int B, int N, int T, int D, int ks, int dtype) {
     if (ks >= 1 && ks % 2 == 1 && T >= 1 && T < ks) {
         set_error("%s: sequence length %d is smaller than kernel_size %d", fn, T, ks);
         return ENATTEN_EINVAL;
     }
-    return check_shape(fn, B, N, T, T, D, ks, dtype);
+    if (ks < 1 || ks % 2 == 0) return check_shape(fn, B, N, 1, T, D, ks, dtype);  // reports it
+    return check_shape(fn, B, N, 1, T, D, 1, dtype);
 }
 
 int enatten1d_fwd(const void *q, const void *k, const void *v, void *o, float *lse, int B,
                   int heads, int T, int D, int kernel_size, int dtype, const int64_t *q_strides,
-                  const int64_t *k_strides, const int64_t *v_strides, float scale,
-                  void *stream) {
+                  const int64_t *k_strides, const int64_t *v_strides, const int64_t *o_strides,
+                  float scale, void *stream) {
     const char *fn = "enatten1d_fwd";
     int rc = check_shape_1d(fn, B, heads, T, D, kernel_size, dtype);
     if (rc) return rc;
@@ -240,11 +209,7 @@ int enatten1d_fwd(const void *q, const void *k, const void *v, void *o, float *l
     if ((rc = view_1d(fn, "q", q, q_strides, heads, T, D, &a.q))) return rc;
     if ((rc = view_1d(fn, "k", k, k_strides, heads, T, D, &a.k))) return rc;
     if ((rc = view_1d(fn, "v", v, v_strides, heads, T, D, &a.v))) return rc;
-    if (!o) {
-        set_error("%s: o is NULL", fn);
-        return ENATTEN_EINVAL;
-    }
-    a.o = o;
+    if ((rc = view_1d(fn, "o", o, o_strides, heads, T, D, &a.o))) return rc;
     a.lse = lse;
     a.s = Shape{B, heads, 1, T, D, 1, kernel_size, scale};  // a 1 x k window on a 1 x T image
     return launch_fwd_simt(a, dtype, static_cast<hipStream_t>(stream));
@@ -257,8 +222,8 @@ size_t enatten1d_bwd_workspace_bytes(int B, int heads, int T) {
 int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,
                   const float *lse, void *dq, void *dk, void *dv, void *workspace, int B,
                   int heads, int T, int D, int kernel_size, int dtype, const int64_t *q_strides,
-                  const int64_t *k_strides, const int64_t *v_strides, float scale,
-                  void *stream) {
+                  const int64_t *k_strides, const int64_t *v_strides, const int64_t *o_strides,
+                  const int64_t *do_strides, float scale, void *stream) {
     const char *fn = "enatten1d_bwd";
     int rc = check_shape_1d(fn, B, heads, T, D, kernel_size, dtype);
     if (rc) return rc;
@@ -266,55 +231,18 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, co
     if ((rc = view_1d(fn, "q", q, q_strides, heads, T, D, &a.q))) return rc;
     if ((rc = view_1d(fn, "k", k, k_strides, heads, T, D, &a.k))) return rc;
     if ((rc = view_1d(fn, "v", v, v_strides, heads, T, D, &a.v))) return rc;
-    if (!o || !d_o || !lse || !dq || !dk || !dv || !workspace) {
-        set_error("%s: o, d_o, lse, dq, dk, dv and workspace must all be non-NULL", fn);
+    if ((rc = view_1d(fn, "o", o, o_strides, heads, T, D, &a.o))) return rc;
+    if ((rc = view_1d(fn, "d_o", d_o, do_strides, heads, T, D, &a.d_o))) return rc;
+    if (!lse || !dq || !dk || !dv || !workspace) {
+        set_error("%s: lse, dq, dk, dv and workspace must all be non-NULL", fn);
         return ENATTEN_EINVAL;
     }
-    a.o = o; a.d_o = d_o; a.lse = lse;
+    a.lse = lse;
     a.dq = dq; a.dk = dk; a.dv = dv;
     a.delta = static_cast<float *>(workspace);
     a.zinv = a.delta + (size_t)B * heads * T;
     a.s = Shape{B, heads, 1, T, D, 1, kernel_size, scale};
     return launch_bwd_simt(a, dtype, static_cast<hipStream_t>(stream));
-}
-
-int enatten_profile_enable(int on) {
-    const int prev = g_prof_on ? g_prof_period : 0;
-    if (on > 0) {
-        for (auto &ps : g_prof) {
-            ps.used = 0;
-            ps.calls = 0;
-        }
-        g_prof_period = on;
-    }
-    g_prof_on = on > 0;
-    return prev;
-}
-
-int enatten_profile_read(int kernel, int *launches, double *total_ms) {
-    if (kernel < 0 || kernel >= ENATTEN_KERNEL_COUNT || !launches || !total_ms) {
-        set_error("enatten_profile_read: bad arguments");
-        return ENATTEN_EINVAL;
-    }
-    ProfSlot &ps = g_prof[kernel];
-    double sum = 0.0;
-    for (int i = 0; i < ps.used; i++) {
-        float ms = 0.f;
-        if (hipEventSynchronize(ps.recs[i].e1) != hipSuccess ||
-            hipEventElapsedTime(&ms, ps.recs[i].e0, ps.recs[i].e1) != hipSuccess) {
-            set_error("enatten_profile_read: event query failed");
-            return ENATTEN_ELAUNCH;
-        }
-        sum += ms;
-    }
-    *launches = ps.used;
-    *total_ms = sum;
-    return ENATTEN_OK;
-}
-
-const char *enatten_profile_kernel_name(int kernel) {
-    if (kernel < 0 || kernel >= ENATTEN_KERNEL_COUNT) return "";
-    return g_prof[kernel].name;
 }
 
 #pragma GCC visibility pop

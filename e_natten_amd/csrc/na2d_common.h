@@ -22,14 +22,14 @@ struct Shape {
 
 struct FwdArgs {
     View q, k, v;
-    void *o;     // contiguous
+    View o;      // written; same kind of strided view as q, k, v
     float *lse;  // contiguous [B, N, H, W] or nullptr
     Shape s;
 };
 
 struct BwdArgs {
     View q, k, v;
-    const void *o, *d_o;  // contiguous
+    View o, d_o;  // forward output and upstream gradient, strided views like q, k, v
     const float *lse;
     void *dq, *dk, *dv;  // contiguous
     float *delta;        // scratch [B, N, H, W]: sum_j P_j dP_j per query
@@ -61,13 +61,18 @@ struct TileSet {
 
 void set_error(const char *fmt, ...);
 
-// Brackets one kernel launch with HIP events when profiling is enabled.
+// Brackets one kernel launch with HIP events while the timing aid is enabled
+// (enatten_prof.cpp); does nothing, and touches no shared state, while it is off.
 struct ProfScope {
     int slot;
     hipStream_t st;
-    void *rec;
+    hipEvent_t e0, e1;
+    unsigned generation;
+    bool armed;
     ProfScope(int kernel_slot, const char *kernel_name, hipStream_t stream);
     ~ProfScope();
+    ProfScope(const ProfScope &) = delete;
+    ProfScope &operator=(const ProfScope &) = delete;
 };
 
 // general fp32-FMA kernels: any D <= 1024, any odd window, f32 / bf16 / f16

@@ -166,7 +166,8 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
                         o[mt]);
             }
 
-            store_token<BF, D>(static_cast<short *>(a.o) + lq.tok * D, g, o, 1.f / sum, lq.live);
+            store_token<BF, D>(const_cast<short *>(image<short>(a.o, cur)) + lq.qr * a.o.sh + lq.qc * a.o.sw,
+                               g, o, 1.f / sum, lq.live);
             if (lq.live && a.lse && g == 0)
                 a.lse[lq.tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
         }
@@ -222,7 +223,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
             halo_fetch<D, KS>(vst, plan, image<short>(a.v, tl), a.v.sh, a.v.sw, lq.hr0, lq.hc0, s.H, s.W);
         }
         const short *qp = image<short>(a.q, tl) + lq.qr * a.q.sh + lq.qc * a.q.sw + g * 8;
-        const short *gp = static_cast<const short *>(a.d_o) + lq.tok * D + g * 8;
+        const short *gp = image<short>(a.d_o, tl) + lq.qr * a.d_o.sh + lq.qc * a.d_o.sw + g * 8;
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) {
             qnext[ds] = *reinterpret_cast<const s16x8 *>(qp + ds * 32);
@@ -430,12 +431,10 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         const int br = tl.r0 - KS / 2, bc = tl.c0 - KS / 2;
         if constexpr (ROLL) {
             halo_fetch_rows<D, KS>(qst, plan, image<short>(a.q, tl), a.q.sh, a.q.sw, y0, bc, nr, s.H, s.W);
-            halo_fetch_rows<D, KS>(gst, plan, static_cast<const short *>(a.d_o) + img_tok * D,
-                                   (int64_t)s.W * D, D, y0, bc, nr, s.H, s.W);
+            halo_fetch_rows<D, KS>(gst, plan, image<short>(a.d_o, tl), a.d_o.sh, a.d_o.sw, y0, bc, nr, s.H, s.W);
         } else {
             halo_fetch<D, KS>(qst, plan, image<short>(a.q, tl), a.q.sh, a.q.sw, br, bc, s.H, s.W);
-            halo_fetch<D, KS>(gst, plan, static_cast<const short *>(a.d_o) + img_tok * D,
-                              (int64_t)s.W * D, D, br, bc, s.H, s.W);
+            halo_fetch<D, KS>(gst, plan, image<short>(a.d_o, tl), a.d_o.sh, a.d_o.sw, br, bc, s.H, s.W);
         }
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
@@ -601,8 +600,7 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
     auto stage = [&](const KeyBlock &b) __attribute__((always_inline)) {
         const int64_t img_tok = ((int64_t)b.tl.bb * s.N + b.tl.nn) * s.H * (int64_t)s.W;
         halo_fetch<D, KS>(qst, plan, image<short>(a.q, b.tl), a.q.sh, a.q.sw, b.br, b.bc, b.qb, b.cb);
-        halo_fetch<D, KS>(gst, plan, static_cast<const short *>(a.d_o) + img_tok * D,
-                          (int64_t)s.W * D, D, b.br, b.bc, b.qb, b.cb);
+        halo_fetch<D, KS>(gst, plan, image<short>(a.d_o, b.tl), a.d_o.sh, a.d_o.sw, b.br, b.bc, b.qb, b.cb);
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
             const int id = threadIdx.x + i * 256;
@@ -866,8 +864,8 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         const bool fused_pays = nb >= 2048 && nb <= 12288 && tiles_r >= 12 && tiles_c >= 12;
         if (path != ENATTEN_PATH_MFMA_SPLIT && fused_bwd_supported(a) &&
             (path == ENATTEN_PATH_MFMA_FUSED || fused_pays)) {
-            launch_bwd_fused(a, BF, ts, nb, st);
-            return check_launch("enatten2d_bwd");
+            const int rc = launch_bwd_fused(a, BF, ts, nb, st);
+            return rc ? rc : check_launch("enatten2d_bwd");
         }
 
         bool dq_done = false;
@@ -958,8 +956,7 @@ bool mfma_supported(int D, int ks, int dtype) {
 }
 
 int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st) {
-    if (!layout_ok(a.q) || !layout_ok(a.k) || !layout_ok(a.v) ||
-        reinterpret_cast<uintptr_t>(a.o) % 16 != 0)
+    if (!layout_ok(a.q) || !layout_ok(a.k) || !layout_ok(a.v) || !layout_ok(a.o))
         return launch_fwd_simt(a, dtype, st);  // 16-byte loads need aligned rows
     if (dtype == ENATTEN_BF16) {
         ENATTEN_BY_D(fwd_launch, true, a, st)
@@ -972,8 +969,8 @@ int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st) {
 
 int launch_bwd_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st) {
     auto al = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-    if (!layout_ok(a.q) || !layout_ok(a.k) || !layout_ok(a.v) || !al(a.o) || !al(a.d_o) ||
-        !al(a.dq) || !al(a.dk) || !al(a.dv))
+    if (!layout_ok(a.q) || !layout_ok(a.k) || !layout_ok(a.v) || !layout_ok(a.o) ||
+        !layout_ok(a.d_o) || !al(a.dq) || !al(a.dk) || !al(a.dv))
         return launch_bwd_simt(a, dtype, st);
     if (dtype == ENATTEN_BF16) {
         ENATTEN_BY_D(bwd_launch, true, a, path, st)

@@ -171,9 +171,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
 
     // ---- staging: a step moves BR rows x HC columns of the block, all five tensors.
     // Chunk i of this thread is channel chunk tid % CPR of pixel tid / CPR + i * RP of
-    // the step (row-major).  q, k, v rows are laid out like dO and O here (stride W*D
-    // between rows, D between pixels; checked on the host), so one set of offsets
-    // serves all five tensors.
+    // the step (row-major).  Every tensor comes with its own row and pixel strides.
     int stid = tid;  // laundered once per tile, see the tile loop
     auto ch8_of = [&]() __attribute__((always_inline)) { return (stid % G::CPR) * 8; };
     Chunks<F::NL> qst, gst, kst, vst, ost;
@@ -194,20 +192,21 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     // they would hold registers through the math of a whole tile.
     // `side` (a compile-time 0 or 1) is the side of the calling wave: the key-side waves
     // then provably never touch the chunk registers beyond their share.
-    auto fetch = [&](Chunks<F::NL> &reg, const short *img, int y0, int bc, auto nr, auto side)
-                     __attribute__((always_inline)) {
+    auto fetch = [&](Chunks<F::NL> &reg, const View &vw, const Tile &tl, int y0, int bc, auto nr,
+                     auto side) __attribute__((always_inline)) {
         constexpr int NR = decltype(nr)::value;
         constexpr int SIDE = decltype(side)::value;
         constexpr int MINE = SIDE == 0 ? F::q_passes(NR) : F::passes(NR) - F::q_passes(NR);
-        const char *base = reinterpret_cast<const char *>(img);
+        const char *base = reinterpret_cast<const char *>(image<short>(vw, tl));
+        const unsigned sh2 = (unsigned)vw.sh * 2u, sw2 = (unsigned)vw.sw * 2u;
 #pragma unroll
         for (int i = 0; i < MINE; i++) {
             const int pix = step_pixel(i, nr, SIDE);
             if (pix >= 0) {
                 const int y = min(max(y0 + pix / G::HC, 0), s.H - 1);
                 const int x = min(max(bc + pix % G::HC, 0), s.W - 1);
-                const unsigned off =
-                    ((unsigned)y * (unsigned)s.W + (unsigned)x) * (D * 2u) + (unsigned)ch8_of() * 2u;
+                const unsigned off = __umul24((unsigned)y, sh2) + __umul24((unsigned)x, sw2) +
+                                     (unsigned)ch8_of() * 2u;
                 reg.v[i] = *reinterpret_cast<const u32x4 *>(base + off);
             }
         }
@@ -220,18 +219,18 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         constexpr int NR = decltype(nr)::value;
         const int64_t img_tok = ((int64_t)tl.bb * s.N + tl.nn) * s.H * (int64_t)s.W;
         if (part == 0) {
-            fetch(qst, image<short>(a.q, tl), y0, bc, nr, side);
+            fetch(qst, a.q, tl, y0, bc, nr, side);
             const int id = min(stid, NR * G::HC - 1);
             const int y = min(max(y0 + id / G::HC, 0), s.H - 1), x = min(max(bc + id % G::HC, 0), s.W - 1);
             lse_st = a.lse[img_tok + (int64_t)y * s.W + x];
         } else if (part == 1) {
-            fetch(kst, image<short>(a.k, tl), y0, bc, nr, side);
+            fetch(kst, a.k, tl, y0, bc, nr, side);
         } else if (part == 2) {
-            fetch(vst, image<short>(a.v, tl), y0, bc, nr, side);
+            fetch(vst, a.v, tl, y0, bc, nr, side);
         } else if (part == 3) {
-            fetch(gst, static_cast<const short *>(a.d_o) + img_tok * D, y0, bc, nr, side);
+            fetch(gst, a.d_o, tl, y0, bc, nr, side);
         } else {
-            fetch(ost, static_cast<const short *>(a.o) + img_tok * D, y0, bc, nr, side);
+            fetch(ost, a.o, tl, y0, bc, nr, side);
         }
     };
     // registers -> LDS; image row y goes to row slot (y + HALF) % HR
@@ -606,13 +605,14 @@ int fused_launch(const BwdArgs &a, const TileSet &ts, int64_t ntiles, hipStream_
 
 // The fused backward is built for head_dim 128 with kernel_size 5.  It needs image
 // sides that are multiples of 8 (then the block of a tile holds everything the tile
-// needs, also beside the border), q, k, v rows laid out like dO's, and 32-bit byte
-// offsets inside one image.
+// needs, also beside the border) and 32-bit byte offsets inside one image of every
+// input (24-bit row and pixel strides are checked by layout_ok).
 bool fused_bwd_supported(const BwdArgs &a) {
-    auto rows_like_o = [&](const View &v) { return v.sh == (int64_t)a.s.W * a.s.D && v.sw == a.s.D; };
+    auto small = [&](const View &v) {
+        return ((int64_t)a.s.H * v.sh + (int64_t)a.s.W * v.sw + a.s.D) * 2 < ((int64_t)1 << 32);
+    };
     return a.s.D == 128 && a.s.kh == 5 && a.s.kw == 5 && a.s.H % 8 == 0 && a.s.W % 8 == 0 &&
-           rows_like_o(a.q) && rows_like_o(a.k) && rows_like_o(a.v) &&
-           (int64_t)a.s.H * a.s.W * a.s.D < ((int64_t)1 << 30);
+           small(a.q) && small(a.k) && small(a.v) && small(a.o) && small(a.d_o);
 }
 
 // dQ, dK, dV of all tiles in one launch.

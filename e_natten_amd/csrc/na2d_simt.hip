@@ -202,7 +202,7 @@ __global__ __launch_bounds__(256) void fwd_simt(FwdArgs a, int tiles_x, int tile
     if (!pl.live) return;
     const float inv = 1.f / l;
     const int64_t tok = (((int64_t)pl.b * s.N + pl.n) * s.H + pl.x) * s.W + pl.y;
-    T *op = static_cast<T *>(a.o) + tok * s.D;
+    T *op = const_cast<T *>(at<T>(a.o, pl.b, pl.n, pl.x, pl.y));
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         const int d0 = (c * G + pl.lg) * 8;
@@ -223,8 +223,8 @@ __global__ __launch_bounds__(256) void bwd_dq_simt(BwdArgs a, int tiles_x, int t
 
     float qr[CH][8], gr[CH][8], acc[CH][8], pk[CH][8];
     const T *qp = at<T>(a.q, pl.b, pl.n, pl.x, pl.y);
-    const T *gp = static_cast<const T *>(a.d_o) + tok * s.D;
-    const T *op = static_cast<const T *>(a.o) + tok * s.D;
+    const T *gp = at<T>(a.d_o, pl.b, pl.n, pl.x, pl.y);
+    const T *op = at<T>(a.o, pl.b, pl.n, pl.x, pl.y);
     float dpart = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; c++) {
@@ -325,7 +325,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_simt(BwdArgs a, int tiles_x, int
         for (int yi = qy0; yi < qy1; yi++) {
             const int64_t qtok = img + (int64_t)xi * s.W + yi;
             const T *qp = at<T>(a.q, pl.b, pl.n, xi, yi);
-            const T *gp = static_cast<const T *>(a.d_o) + qtok * s.D;
+            const T *gp = at<T>(a.d_o, pl.b, pl.n, xi, yi);
             float qr[CH][8], gr[CH][8];
             A ps = 0;
             float pd = 0.f;

@@ -87,12 +87,15 @@ std::tuple<Tensor, Tensor> na2d_fwd(const Tensor &q_, const Tensor &k_, const Te
     const c10::DeviceGuard guard(q_.device());
     const Tensor q = kernel_layout(q_), k = kernel_layout(k_), v = kernel_layout(v_);
     const int B = q.size(0), N = q.size(1), H = q.size(2), W = q.size(3), D = q.size(4);
-    Tensor o = at::empty({B, N, H, W, D}, q.options());
+    // like the reference's zeros_like(Q) (e_natten/triton.py:502) the output takes the
+    // memory order of q
+    Tensor o = kernel_layout(at::empty_like(q));
     Tensor lse = at::empty({B, N, H, W}, q.options().dtype(at::kFloat));
     check_rc(enatten2d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                            lse.data_ptr<float>(), B, N, H, W, D, (int)ks, dtype_code(q),
                            q.strides().data(), k.strides().data(), v.strides().data(),
-                           (float)scale, c10::hip::getCurrentHIPStream().stream()));
+                           o.strides().data(), (float)scale,
+                           c10::hip::getCurrentHIPStream().stream()));
     return {o, lse};
 }
 
@@ -103,7 +106,7 @@ std::tuple<Tensor, Tensor, Tensor> na2d_bwd(const Tensor &q_, const Tensor &k_, 
     check_bwd_extras("enatten::na2d_bwd", q_, o_, d_o_);
     const c10::DeviceGuard guard(q_.device());
     const Tensor q = kernel_layout(q_), k = kernel_layout(k_), v = kernel_layout(v_);
-    const Tensor o = o_.contiguous(), d_o = d_o_.contiguous(), lse = lse_.contiguous();
+    const Tensor o = kernel_layout(o_), d_o = kernel_layout(d_o_), lse = lse_.contiguous();
     const int B = q.size(0), N = q.size(1), H = q.size(2), W = q.size(3), D = q.size(4);
     Tensor dq = at::empty({B, N, H, W, D}, q.options());
     Tensor dk = at::empty_like(dq), dv = at::empty_like(dq);
@@ -113,7 +116,8 @@ std::tuple<Tensor, Tensor, Tensor> na2d_bwd(const Tensor &q_, const Tensor &k_, 
                            lse.data_ptr<float>(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                            ws.data_ptr(), B, N, H, W, D, (int)ks, dtype_code(q),
                            q.strides().data(), k.strides().data(), v.strides().data(),
-                           (float)scale, c10::hip::getCurrentHIPStream().stream()));
+                           o.strides().data(), d_o.strides().data(), (float)scale,
+                           c10::hip::getCurrentHIPStream().stream()));
     return {dq, dk, dv};
 }
 
@@ -123,12 +127,13 @@ std::tuple<Tensor, Tensor> na1d_fwd(const Tensor &q_, const Tensor &k_, const Te
     const c10::DeviceGuard guard(q_.device());
     const Tensor q = kernel_layout(q_), k = kernel_layout(k_), v = kernel_layout(v_);
     const int B = q.size(0), N = q.size(1), T = q.size(2), D = q.size(3);
-    Tensor o = at::empty({B, N, T, D}, q.options());
+    Tensor o = kernel_layout(at::empty_like(q));
     Tensor lse = at::empty({B, N, T}, q.options().dtype(at::kFloat));
     check_rc(enatten1d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                            lse.data_ptr<float>(), B, N, T, D, (int)ks, dtype_code(q),
                            q.strides().data(), k.strides().data(), v.strides().data(),
-                           (float)scale, c10::hip::getCurrentHIPStream().stream()));
+                           o.strides().data(), (float)scale,
+                           c10::hip::getCurrentHIPStream().stream()));
     return {o, lse};
 }
 
@@ -139,7 +144,7 @@ std::tuple<Tensor, Tensor, Tensor> na1d_bwd(const Tensor &q_, const Tensor &k_, 
     check_bwd_extras("enatten::na1d_bwd", q_, o_, d_o_);
     const c10::DeviceGuard guard(q_.device());
     const Tensor q = kernel_layout(q_), k = kernel_layout(k_), v = kernel_layout(v_);
-    const Tensor o = o_.contiguous(), d_o = d_o_.contiguous(), lse = lse_.contiguous();
+    const Tensor o = kernel_layout(o_), d_o = kernel_layout(d_o_), lse = lse_.contiguous();
     const int B = q.size(0), N = q.size(1), T = q.size(2), D = q.size(3);
     Tensor dq = at::empty({B, N, T, D}, q.options());
     Tensor dk = at::empty_like(dq), dv = at::empty_like(dq);
@@ -148,7 +153,8 @@ std::tuple<Tensor, Tensor, Tensor> na1d_bwd(const Tensor &q_, const Tensor &k_, 
     check_rc(enatten1d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(),
                            lse.data_ptr<float>(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                            ws.data_ptr(), B, N, T, D, (int)ks, dtype_code(q), q.strides().data(),
-                           k.strides().data(), v.strides().data(), (float)scale,
+                           k.strides().data(), v.strides().data(), o.strides().data(),
+                           d_o.strides().data(), (float)scale,
                            c10::hip::getCurrentHIPStream().stream()));
     return {dq, dk, dv};
 }

@@ -58,8 +58,8 @@ def _validate(q, k, v, kernel_size: int, ndim: int = 5) -> None:
 
 
 def _kernel_layout(t: torch.Tensor) -> torch.Tensor:
-    """The kernels take any strides on the leading axes but need unit stride on
-    the channel axis and no negative strides."""
+    """The kernels take any strides on the leading axes (of q, k, v, o and dO alike)
+    but need unit stride on the channel axis; torch has no negative strides."""
     if t.stride(-1) != 1 and t.shape[-1] != 1:
         return t.contiguous()
     return t
@@ -71,12 +71,10 @@ def _require_gpu(t: torch.Tensor, what: str) -> None:
 
 
 def _stream_of(t: torch.Tensor) -> int:
-    """Raw HIP stream that torch orders work on for the tensor's device; that
-    device is made current only if it is not already."""
-    idx = t.device.index
-    if idx is not None and idx != torch.cuda.current_device():
-        torch.cuda.set_device(idx)
-    return torch.cuda.current_stream().cuda_stream
+    """Raw HIP stream that torch orders work on for the tensor's device.  Called
+    with that device current (the callers hold ``torch.cuda.device(t.device)``,
+    which puts the previous device back when the call is over)."""
+    return torch.cuda.current_stream(t.device).cuda_stream
 
 
 def _check(rc: int) -> None:
@@ -91,12 +89,16 @@ def _fwd_impl(q, k, v, kernel_size: int, scale: float):
     lib = _lib.load()
     q, k, v = (_kernel_layout(t) for t in (q, k, v))
     B, N, H, W, D = q.shape
-    o = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
-    lse = torch.empty((B, N, H, W), dtype=torch.float32, device=q.device)
-    _check(lib.enatten2d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                             lse.data_ptr(), B, N, H, W, D, kernel_size, _DTYPES[q.dtype],
-                             _lib.strides4(q), _lib.strides4(k), _lib.strides4(v),
-                             float(scale), _stream_of(q)))
+    with torch.cuda.device(q.device):
+        # like the reference's zeros_like(Q) (e_natten/triton.py:502), the output takes
+        # the memory order of q: for q sliced out of a [B, H, W, 3, heads, d] projection
+        # that is [B, H, W, heads, d], which the following merge of heads needs
+        o = _kernel_layout(torch.empty_like(q))
+        lse = torch.empty((B, N, H, W), dtype=torch.float32, device=q.device)
+        _check(lib.enatten2d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                 lse.data_ptr(), B, N, H, W, D, kernel_size, _DTYPES[q.dtype],
+                                 _lib.strides4(q), _lib.strides4(k), _lib.strides4(v),
+                                 _lib.strides4(o), float(scale), _stream_of(q)))
     return o, lse
 
 
@@ -108,18 +110,20 @@ def _bwd_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
     if d_o.dtype != q.dtype or o.dtype != q.dtype:
         raise ValueError("o and d_o must have the dtype of q")
     lib = _lib.load()
-    q, k, v = (_kernel_layout(t) for t in (q, k, v))
-    o, d_o, lse = o.contiguous(), d_o.contiguous(), lse.contiguous()
+    q, k, v, o, d_o = (_kernel_layout(t) for t in (q, k, v, o, d_o))
+    lse = lse.contiguous()
     B, N, H, W, D = q.shape
-    dq = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
-    dk, dv = torch.empty_like(dq), torch.empty_like(dq)
-    ws = torch.empty(lib.enatten2d_bwd_workspace_bytes(B, N, H, W), dtype=torch.uint8,
-                     device=q.device)
-    _check(lib.enatten2d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                             d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                             dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, kernel_size,
-                             _DTYPES[q.dtype], _lib.strides4(q), _lib.strides4(k),
-                             _lib.strides4(v), float(scale), _stream_of(q)))
+    with torch.cuda.device(q.device):
+        dq = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
+        dk, dv = torch.empty_like(dq), torch.empty_like(dq)
+        ws = torch.empty(lib.enatten2d_bwd_workspace_bytes(B, N, H, W), dtype=torch.uint8,
+                         device=q.device)
+        _check(lib.enatten2d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                 d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                 dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, kernel_size,
+                                 _DTYPES[q.dtype], _lib.strides4(q), _lib.strides4(k),
+                                 _lib.strides4(v), _lib.strides4(o), _lib.strides4(d_o),
+                                 float(scale), _stream_of(q)))
     return dq, dk, dv
 
 
@@ -129,12 +133,13 @@ def _fwd1d_impl(q, k, v, kernel_size: int, scale: float):
     lib = _lib.load()
     q, k, v = (_kernel_layout(t) for t in (q, k, v))
     B, N, T, D = q.shape
-    o = torch.empty((B, N, T, D), dtype=q.dtype, device=q.device)
-    lse = torch.empty((B, N, T), dtype=torch.float32, device=q.device)
-    _check(lib.enatten1d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                             lse.data_ptr(), B, N, T, D, kernel_size, _DTYPES[q.dtype],
-                             _lib.strides3(q), _lib.strides3(k), _lib.strides3(v),
-                             float(scale), _stream_of(q)))
+    with torch.cuda.device(q.device):
+        o = _kernel_layout(torch.empty_like(q))
+        lse = torch.empty((B, N, T), dtype=torch.float32, device=q.device)
+        _check(lib.enatten1d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                 lse.data_ptr(), B, N, T, D, kernel_size, _DTYPES[q.dtype],
+                                 _lib.strides3(q), _lib.strides3(k), _lib.strides3(v),
+                                 _lib.strides3(o), float(scale), _stream_of(q)))
     return o, lse
 
 
@@ -146,18 +151,20 @@ def _bwd1d_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
     if d_o.dtype != q.dtype or o.dtype != q.dtype:
         raise ValueError("o and d_o must have the dtype of q")
     lib = _lib.load()
-    q, k, v = (_kernel_layout(t) for t in (q, k, v))
-    o, d_o, lse = o.contiguous(), d_o.contiguous(), lse.contiguous()
+    q, k, v, o, d_o = (_kernel_layout(t) for t in (q, k, v, o, d_o))
+    lse = lse.contiguous()
     B, N, T, D = q.shape
-    dq = torch.empty((B, N, T, D), dtype=q.dtype, device=q.device)
-    dk, dv = torch.empty_like(dq), torch.empty_like(dq)
-    ws = torch.empty(lib.enatten1d_bwd_workspace_bytes(B, N, T), dtype=torch.uint8,
-                     device=q.device)
-    _check(lib.enatten1d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                             d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                             dv.data_ptr(), ws.data_ptr(), B, N, T, D, kernel_size,
-                             _DTYPES[q.dtype], _lib.strides3(q), _lib.strides3(k),
-                             _lib.strides3(v), float(scale), _stream_of(q)))
+    with torch.cuda.device(q.device):
+        dq = torch.empty((B, N, T, D), dtype=q.dtype, device=q.device)
+        dk, dv = torch.empty_like(dq), torch.empty_like(dq)
+        ws = torch.empty(lib.enatten1d_bwd_workspace_bytes(B, N, T), dtype=torch.uint8,
+                         device=q.device)
+        _check(lib.enatten1d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                 d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                 dv.data_ptr(), ws.data_ptr(), B, N, T, D, kernel_size,
+                                 _DTYPES[q.dtype], _lib.strides3(q), _lib.strides3(k),
+                                 _lib.strides3(v), _lib.strides3(o), _lib.strides3(d_o),
+                                 float(scale), _stream_of(q)))
     return dq, dk, dv
 
 
@@ -171,7 +178,10 @@ def _load_native_binding() -> bool:
         return False
     if not (os.path.exists(path) and os.path.exists(_lib.LIB_PATH)):
         return False
-    _lib.load()
+    try:
+        _lib.load()
+    except ImportError:  # stale or broken build: every call will say so; importing must
+        return False     # still work, or `python -m e_natten_amd.build` could not run
     try:
         torch.ops.load_library(path)
     except OSError as e:  # built against another torch: keep working through Python

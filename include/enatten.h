@@ -7,11 +7,14 @@
  * code and enatten_last_error() describes it (per calling thread).
  *
  * Tensor layout: [B, heads, H, W, D] as in the reference
- * (e_natten/triton.py:489-518).  The last axis has stride 1.  q, k and v may be
- * strided views: their element strides for the (batch, head, row, column) axes
- * are passed as int64_t[4]; NULL means contiguous.  All other tensors are
- * contiguous.  The logits are q.k * scale; the reference applies no scale
- * (e_natten/triton.py:280), so drop-in callers pass 1.0f.
+ * (e_natten/triton.py:489-518).  The last axis has stride 1.  q, k, v, the forward
+ * output o and the upstream gradient d_o may be strided views, as in the reference,
+ * which passes the strides of each of them to its kernels
+ * (e_natten/triton.py:509-512, :539-545): their element strides for the (batch,
+ * head, row, column) axes are passed as int64_t[4]; NULL means contiguous.  The
+ * gradients dq, dk, dv, the log-sum-exp and the workspace are contiguous.  The logits
+ * are q.k * scale; the reference applies no scale (e_natten/triton.py:280), so
+ * drop-in callers pass 1.0f.
  */
 #ifndef ENATTEN_H
 #define ENATTEN_H
@@ -23,7 +26,7 @@
 extern "C" {
 #endif
 
-#define ENATTEN_ABI_VERSION 1
+#define ENATTEN_ABI_VERSION 2
 
 /* element types of q, k, v, o and the gradients */
 enum { ENATTEN_F32 = 0, ENATTEN_BF16 = 1, ENATTEN_F16 = 2 };
@@ -70,7 +73,9 @@ int enatten_set_path(int path);
  * (e_natten/triton.py:507-513; per-query math triton.py:242-302, CPU statement
  * e_natten/pytorch.py:178-202).
  *
- *   o   [B, heads, H, W, D]  dtype, contiguous, fully overwritten
+ *   o   [B, heads, H, W, D]  dtype, every element overwritten; o_strides lets the
+ *                            caller have it written straight into, say, a
+ *                            [B, H, W, heads, D] buffer
  *   lse [B, heads, H, W]     float32 natural-log sum-exp of each query's scaled
  *                            logits, contiguous; may be NULL if no backward
  *                            will follow
@@ -79,7 +84,8 @@ int enatten_set_path(int path);
 int enatten2d_fwd(const void *q, const void *k, const void *v, void *o, float *lse,
                   int B, int heads, int H, int W, int D, int kernel_size, int dtype,
                   const int64_t *q_strides, const int64_t *k_strides,
-                  const int64_t *v_strides, float scale, void *stream);
+                  const int64_t *v_strides, const int64_t *o_strides, float scale,
+                  void *stream);
 
 /*
  * Bytes of device scratch enatten2d_bwd needs (two float32 per query).
@@ -94,7 +100,8 @@ size_t enatten2d_bwd_workspace_bytes(int B, int heads, int H, int W);
  * key's inverse neighbourhood (pytorch.py:261-270), not by atomics, so results
  * are deterministic and the outputs need no zero-fill.
  *
- *   o, d_o      [B, heads, H, W, D] dtype, contiguous (forward output, upstream grad)
+ *   o, d_o      [B, heads, H, W, D] dtype (forward output, upstream gradient), read
+ *               through o_strides / do_strides
  *   lse         as written by enatten2d_fwd with the same scale
  *   dq, dk, dv  [B, heads, H, W, D] dtype, contiguous, fully overwritten
  *   workspace   enatten2d_bwd_workspace_bytes() bytes of device memory
@@ -103,7 +110,8 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o,
                   const void *d_o, const float *lse, void *dq, void *dk, void *dv,
                   void *workspace, int B, int heads, int H, int W, int D,
                   int kernel_size, int dtype, const int64_t *q_strides,
-                  const int64_t *k_strides, const int64_t *v_strides, float scale,
+                  const int64_t *k_strides, const int64_t *v_strides,
+                  const int64_t *o_strides, const int64_t *do_strides, float scale,
                   void *stream);
 
 /*
@@ -117,26 +125,30 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o,
 int enatten1d_fwd(const void *q, const void *k, const void *v, void *o, float *lse,
                   int B, int heads, int T, int D, int kernel_size, int dtype,
                   const int64_t *q_strides, const int64_t *k_strides,
-                  const int64_t *v_strides, float scale, void *stream);
+                  const int64_t *v_strides, const int64_t *o_strides, float scale,
+                  void *stream);
 size_t enatten1d_bwd_workspace_bytes(int B, int heads, int T);
 int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o,
                   const void *d_o, const float *lse, void *dq, void *dk, void *dv,
                   void *workspace, int B, int heads, int T, int D, int kernel_size,
                   int dtype, const int64_t *q_strides, const int64_t *k_strides,
-                  const int64_t *v_strides, float scale, void *stream);
+                  const int64_t *v_strides, const int64_t *o_strides,
+                  const int64_t *do_strides, float scale, void *stream);
 
 /*
  * Per-kernel timing aid for benchmarks (no counterpart in the reference, whose
  * bench.py:28,59 times whole calls with triton.testing.do_bench).  While
  * enabled, kernels this library launches are bracketed by HIP events on the
- * launch stream.  enatten_profile_enable(n), n >= 1, clears the records and
+ * launch stream.  enatten_profile_enable(n), n >= 1, clears the figures and
  * times every n-th launch of each kernel (an event record costs a few
  * microseconds of queue time, so sampling keeps the timed loop undisturbed);
- * enatten_profile_enable(0) stops; the return value is the previous setting.
- * enatten_profile_read waits for the recorded events of one kernel and returns
- * how many launches were timed and their summed duration.  At most 8192 launches
- * per kernel are recorded between two enables.  Not thread-safe; leave it off in
- * production.
+ * enatten_profile_enable(0) stops, waits for the recorded events, keeps their
+ * durations and destroys them, so no HIP object is left behind; the return value
+ * is the previous setting.  enatten_profile_read returns how many launches of one
+ * kernel were timed and their summed duration (it also waits for and collects
+ * what has been recorded so far).  At most 8192 launches per kernel are timed
+ * between two enables.  Safe to call while other threads launch; while it is off
+ * a launch reads one flag and nothing else.
  */
 enum { ENATTEN_KERNEL_FWD = 0, ENATTEN_KERNEL_BWD_DQ = 1, ENATTEN_KERNEL_BWD_DKDV = 2,
        ENATTEN_KERNEL_BWD_FUSED = 3, ENATTEN_KERNEL_COUNT = 4 };

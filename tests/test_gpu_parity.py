@@ -175,6 +175,155 @@ def test_strided_qkv_views(path):
     assert_close(got, (ref[0], ref[2], ref[3], ref[4]), BF, "strided")
 
 
+@pytest.mark.parametrize("D,ks,H,W", [(64, 5, 20, 24), (128, 5, 24, 32), (32, 7, 16, 20), (48, 3, 9, 10)])
+def test_projection_layout_without_copies(D, ks, H, W, path):
+    # A block's layouts either side of the operator: q, k, v are views of the fused
+    # projection [B, H, W, 3, heads, d]; the output comes back in the memory order of
+    # q, [B, H, W, heads, d], so merging the heads is a view; the upstream gradient
+    # arrives in that order too.  None of the five tensors is copied on the way (the
+    # allocator sees nothing but the outputs and the workspace), and the fused backward
+    # (D = 128, sides multiples of 8) takes the strided rows as they are.
+    from e_natten_amd import natten2d
+    B, N = 2, 4
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(B, H, W, 3, N, D, generator=g).to(BF)
+    d_y = torch.randn(B, H, W, N * D, generator=g).to(BF)
+    q, k, v = (qkv[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+    d_o = d_y.view(B, H, W, N, D).permute(0, 3, 1, 2, 4)
+    ref = oracle_all(q.contiguous(), k.contiguous(), v.contiguous(), d_o.contiguous(), ks, 1.0, small=True)
+    fused = qkv.cuda().requires_grad_(True)
+    qg, kg, vg = (fused[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+    d_y = d_y.cuda()
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    o = natten2d(qg, kg, vg, ks)
+    assert o.permute(0, 2, 3, 1, 4).is_contiguous(), "O is not in the memory order of q"
+    y = o.permute(0, 2, 3, 1, 4).reshape(B, H, W, N * D)
+    assert y.data_ptr() == o.data_ptr(), "merging the heads copied O"
+    y.backward(d_y)
+    torch.cuda.synchronize()
+    # forward: o, lse; backward: dq, dk, dv, workspace, and autograd's gradient of the
+    # projection with the three slices it accumulates: ten blocks at most
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] - before <= 10
+    grads = fused.grad.cpu()
+    got = (o.detach().cpu(),) + tuple(grads[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+    assert_close(got, (ref[0], ref[2], ref[3], ref[4]), BF, "projection layout D=%d" % D)
+
+
+def test_fused_backward_takes_strided_rows(_lib):
+    # the fused backward, forced, on views of a [B, H, W, 3, heads, d] projection and an
+    # upstream gradient in [B, H, W, heads, d] order
+    from e_natten_amd import natten2d
+    from e_natten_amd._lib import PATH_MFMA_FUSED
+    B, N, H, W, D, ks = 2, 3, 40, 32, 128, 5
+    g = torch.Generator().manual_seed(6)
+    qkv = torch.randn(B, H, W, 3, N, D, generator=g).to(BF)
+    d_y = torch.randn(B, H, W, N, D, generator=g).to(BF)
+    q, k, v = (qkv[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+    ref = oracle_all(q.contiguous(), k.contiguous(), v.contiguous(),
+                     d_y.permute(0, 3, 1, 2, 4).contiguous(), ks, 1.0, small=True)
+    prev = _lib.enatten_set_path(PATH_MFMA_FUSED)
+    try:
+        fused = qkv.cuda().requires_grad_(True)
+        qg, kg, vg = (fused[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+        o = natten2d(qg, kg, vg, ks)
+        o.backward(d_y.cuda().permute(0, 3, 1, 2, 4))
+        torch.cuda.synchronize()
+    finally:
+        _lib.enatten_set_path(prev)
+    grads = fused.grad.cpu()
+    got = (o.detach().cpu(),) + tuple(grads[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+    assert_close(got, (ref[0], ref[2], ref[3], ref[4]), BF, "fused backward, strided rows")
+
+
+@pytest.mark.parametrize("shape,ks", [((2, 4, 16, 24, 128), 5), ((1, 2, 20, 20, 64), 7)])
+def test_output_written_into_callers_layout(shape, ks, _lib):
+    # straight through the C ABI: O is written into a [B, H, W, heads, D] buffer through
+    # o_strides and read back from there by the backward, dO is read through do_strides
+    from e_natten_amd import _lib as L
+    import ctypes
+    B, N, H, W, D = shape
+    q, k, v, g = make_inputs(shape, BF, 9)
+    ref = oracle_all(q, k, v, g, ks, small=True)
+    dev = torch.device("cuda:0")
+    qd, kd, vd = (t.to(dev) for t in (q, k, v))
+    o_buf = torch.full((B, H, W, N, D), float("nan"), dtype=BF, device=dev)
+    g_buf = g.permute(0, 2, 3, 1, 4).contiguous().to(dev)          # [B, H, W, heads, D]
+    o_view, g_view = o_buf.permute(0, 3, 1, 2, 4), g_buf.permute(0, 3, 1, 2, 4)
+    lse = torch.empty((B, N, H, W), dtype=torch.float32, device=dev)
+    dq, dk, dv = (torch.full(shape, float("nan"), dtype=BF, device=dev) for _ in range(3))
+    ws = torch.empty(_lib.enatten2d_bwd_workspace_bytes(B, N, H, W), dtype=torch.uint8, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    so, sg = L.strides4(o_view), L.strides4(g_view)
+    rc = _lib.enatten2d_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o_buf.data_ptr(),
+                            lse.data_ptr(), B, N, H, W, D, ks, L.BF16, None, None, None, so, 1.0, st)
+    assert rc == 0, L.last_error()
+    rc = _lib.enatten2d_bwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o_buf.data_ptr(),
+                            g_buf.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                            dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, ks, L.BF16, None, None,
+                            None, so, sg, 1.0, st)
+    assert rc == 0, L.last_error()
+    torch.cuda.synchronize()
+    got = (o_view.cpu(), dq.cpu(), dk.cpu(), dv.cpu())
+    assert_close(got, (ref[0], ref[2], ref[3], ref[4]), BF, "O in the caller's layout")
+
+
+@pytest.mark.parametrize("D,ks", [(128, 5), (64, 7), (32, 3)])
+def test_misaligned_views_take_the_general_kernels(D, ks, _lib):
+    # head dims the matrix-core kernels serve, but as views whose rows are not 16-byte
+    # aligned (channels 4..D+4 of a wider tensor, strides that are no multiples of 8):
+    # the launchers route them to the general kernels with scalar loads
+    from e_natten_amd import natten2d
+    shape = (1, 2, 12, 14, D)
+    q, k, v, g = make_inputs(shape, BF, 13)
+    ref = oracle_all(q, k, v, g, ks, small=True)
+    dev = torch.device("cuda:0")
+    wide = [torch.zeros(shape[:-1] + (D + 12,), dtype=BF, device=dev) for _ in range(4)]
+    views = []
+    for buf, t in zip(wide, (q, k, v, g)):
+        view = buf[..., 4:D + 4]
+        view.copy_(t.to(dev))
+        views.append(view)
+    assert all(t.data_ptr() % 16 != 0 and t.stride(3) % 8 != 0 for t in views)
+    qg, kg, vg = (t.requires_grad_(True) for t in views[:3])
+    o = natten2d(qg, kg, vg, ks)
+    o.backward(views[3])
+    torch.cuda.synchronize()
+    got = tuple(t.detach().cpu() for t in (o, qg.grad, kg.grad, vg.grad))
+    assert_close(got, (ref[0], ref[2], ref[3], ref[4]), BF, "misaligned D=%d" % D)
+
+
+def test_timing_aid_over_several_configurations(_lib):
+    # the per-kernel event timing, switched on and off around several configurations in
+    # one process, with the forward on this thread and the backward on the autograd
+    # engine's thread: every timed launch is read back, and nothing is left recording
+    import ctypes
+    from e_natten_amd import natten2d
+    cases = [((2, 2, 32, 32, 128), BF, 5), ((1, 2, 16, 16, 32), F32, 3), ((2, 4, 28, 28, 32), BF, 7),
+             ((1, 2, 40, 40, 64), BF, 13)]
+    for shape, dtype, ks in cases:
+        q, k, v, g = (t.cuda() for t in make_inputs(shape, dtype, 1))
+        q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
+        assert _lib.enatten_profile_enable(2) == 0
+        for _ in range(6):
+            natten2d(q, k, v, ks).backward(g)
+        assert _lib.enatten_profile_enable(0) == 2
+        n, ms = ctypes.c_int(), ctypes.c_double()
+        seen = {}
+        for slot in range(4):
+            assert _lib.enatten_profile_read(slot, ctypes.byref(n), ctypes.byref(ms)) == 0
+            if n.value:
+                seen[_lib.enatten_profile_kernel_name(slot).decode()] = (n.value, ms.value)
+        assert any(name.startswith("fwd") for name in seen), seen
+        assert all(cnt == 3 and 0.0 < t < 1e3 for cnt, t in seen.values()), seen
+    # off again: launches are not recorded
+    natten2d(q, k, v, ks).backward(g)
+    torch.cuda.synchronize()
+    n, ms = ctypes.c_int(), ctypes.c_double()
+    _lib.enatten_profile_read(0, ctypes.byref(n), ctypes.byref(ms))
+    assert n.value == 3
+
+
 def test_native_binding_is_what_runs(_lib):
     # natten2d goes through the C++ torch binding (no Python in forward or backward);
     # both bindings give bit-identical results; views, no-grad calls and inputs that

@@ -1,6 +1,7 @@
 """Host side and C-ABI surface, without a GPU: the library loads, exports every
 symbol the header declares, validates arguments before touching the device, and
 the Python entry points mirror the reference's signature."""
+import ctypes
 import inspect
 import os
 import re
@@ -29,13 +30,13 @@ def test_library_exports_every_declared_symbol(lib):
     for n in names:
         assert hasattr(lib, n), "libenatten.so does not export %s" % n
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.enatten_abi_version() == 1
+    assert lib.enatten_abi_version() == _lib.ABI_VERSION == 2
 
 
 def test_c_abi_validates_before_launch(lib):
     from e_natten_amd import _lib
     f = lambda ks, H=8, W=8, D=16, dt=0, q=1: lib.enatten2d_fwd(
-        q, 1, 1, 1, None, 1, 1, H, W, D, ks, dt, None, None, None, 1.0, None)
+        q, 1, 1, 1, None, 1, 1, H, W, D, ks, dt, None, None, None, None, 1.0, None)
     assert f(4) == 1 and "odd" in _lib.last_error()
     assert f(-1) == 1
     assert f(9) == 1 and "smaller" in _lib.last_error()
@@ -43,7 +44,14 @@ def test_c_abi_validates_before_launch(lib):
     assert f(3, D=0) == 1
     assert f(3, q=None) == 1 and "NULL" in _lib.last_error()
     assert lib.enatten2d_bwd(1, 1, 1, 1, 1, None, 1, 1, 1, 1, 1, 1, 8, 8, 16, 3, 0,
-                             None, None, None, 1.0, None) == 1
+                             None, None, None, None, None, 1.0, None) == 1
+    # negative strides are refused for every strided tensor, the output included
+    neg = (ctypes.c_int64 * 4)(1024, 512, -128, 16)
+    assert lib.enatten2d_fwd(1, 1, 1, 1, None, 1, 1, 8, 8, 16, 3, 0, None, None, None, neg,
+                             1.0, None) == 1 and "negative stride for o" in _lib.last_error()
+    # more than 2^40 elements: refused as unsupported, before any pointer is looked at
+    assert lib.enatten2d_fwd(None, 1, 1, 1, None, 1 << 12, 1 << 12, 1 << 12, 1 << 12, 1024, 3, 0,
+                             None, None, None, None, 1.0, None) == 2
     assert lib.enatten2d_bwd_workspace_bytes(2, 3, 4, 5) == 2 * 3 * 4 * 5 * 8
     assert lib.enatten2d_bwd_workspace_bytes(0, 3, 4, 5) == 0
 
@@ -128,10 +136,18 @@ def test_1d_surface_and_validation(lib):
     with pytest.raises(RuntimeError, match="no CPU path"):
         natten1d(q, q, q, 3)
     f = lambda ks, T=8: lib.enatten1d_fwd(1, 1, 1, 1, None, 1, 1, T, 16, ks, 0, None, None,
-                                          None, 1.0, None)
+                                          None, None, 1.0, None)
     assert f(4) == 1 and "odd" in _lib.last_error()
     assert f(9) == 1 and "smaller" in _lib.last_error()
     assert lib.enatten1d_bwd_workspace_bytes(2, 3, 10) == 2 * 3 * 10 * 8
+    # The size limit is on B * heads * T * D elements, not on a T x T image: long
+    # sequences pass it and fail on the NULL pointer that follows (nothing is launched).
+    for B, N, T, D in ((8, 8, 16384, 128), (1, 8, 131072, 64), (1, 1, 1 << 22, 64)):
+        rc = lib.enatten1d_fwd(None, 1, 1, 1, None, B, N, T, D, 7, 1, None, None, None, None,
+                               1.0, None)
+        assert rc == 1 and "q is NULL" in _lib.last_error(), (B, N, T, D, _lib.last_error())
+    assert lib.enatten1d_fwd(None, 1, 1, 1, None, 1 << 10, 1 << 10, 1 << 20, 1024, 7, 1, None,
+                             None, None, None, 1.0, None) == 2
 
 
 def test_python_validation_without_gpu():
