@@ -10,6 +10,7 @@ LIB_PATH = os.path.join(_HERE, "libenatten.so")
 
 ABI_VERSION = 2  # ENATTEN_ABI_VERSION of include/enatten.h
 F32, BF16, F16 = 0, 1, 2
+STATIC_BWD_MAX_QUERIES = 1 << 20
 PATH_NONE, PATH_SIMT, PATH_MFMA, PATH_MFMA_FUSED, PATH_MFMA_SPLIT = 0, 1, 2, 3, 4
 
 _lock = threading.Lock()
@@ -28,6 +29,7 @@ SIGNATURES = {
     "enatten2d_fwd": (_i, [_vp] * 5 + [_i] * 7 + [_sp] * 4 + [ctypes.c_float, _vp]),
     "enatten2d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 4),
     "enatten2d_bwd": (_i, [_vp] * 10 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
+    "enatten2d_bwd_static": (_i, [_vp] * 9 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
     "enatten1d_fwd": (_i, [_vp] * 5 + [_i] * 6 + [_sp] * 4 + [ctypes.c_float, _vp]),
     "enatten1d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 3),
     "enatten1d_bwd": (_i, [_vp] * 10 + [_i] * 6 + [_sp] * 5 + [ctypes.c_float, _vp]),
@@ -49,11 +51,14 @@ def load() -> ctypes.CDLL:
                     "%s is missing: build it with `python -m e_natten_amd.build` "
                     "(needs hipcc; cross-compiles for gfx950 without a GPU)" % LIB_PATH)
             lib = ctypes.CDLL(LIB_PATH)
+            stale = "%s is stale (%%s): rebuild it with `python -m e_natten_amd.build`" % LIB_PATH
             for name, (res, args) in SIGNATURES.items():
-                fn = getattr(lib, name)
+                fn = getattr(lib, name, None)
+                if fn is None:
+                    raise ImportError(stale % ("it does not export %s" % name))
                 fn.restype, fn.argtypes = res, args
             if lib.enatten_abi_version() != ABI_VERSION:
-                raise ImportError("libenatten.so has an unexpected ABI version")
+                raise ImportError(stale % "unexpected ABI version")
             _lib = lib
     return _lib
 

@@ -32,8 +32,18 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
-def _compile(src: str) -> str:
+def _up_to_date(src: str, obj: str) -> bool:
+    if not os.path.exists(obj):
+        return False
+    deps = [os.path.join(CSRC, src), os.path.join(ROOT, "include", "enatten.h")]
+    deps += [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    return all(os.path.getmtime(d) <= os.path.getmtime(obj) for d in deps)
+
+
+def _compile(src: str, incremental: bool = False) -> str:
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    if incremental and _up_to_date(src, obj):
+        return obj
     cmd = [_hipcc(), *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -62,22 +72,26 @@ def _build_torch_shim() -> str:
     return TORCH_LIB
 
 
-def build(verbose: bool = False) -> str:
-    """Compile every source and link libenatten.so and the torch binding; returns
-    the path of libenatten.so."""
+def build(verbose: bool = False, incremental: bool = False) -> str:
+    """Compile every source (with `incremental`, only those older than their object
+    file's inputs) and link libenatten.so and the torch binding; returns the path of
+    libenatten.so."""
     os.makedirs(OBJ, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
-        objs = list(ex.map(_compile, SOURCES))
+        objs = list(ex.map(lambda src: _compile(src, incremental), SOURCES))
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s" % r.stderr[-4000:])
-    _build_torch_shim()
+    shim_deps = [os.path.join(CSRC, "torch_shim.cpp"), os.path.join(ROOT, "include", "enatten.h")]
+    if not (incremental and os.path.exists(TORCH_LIB) and
+            all(os.path.getmtime(d) <= os.path.getmtime(TORCH_LIB) for d in shim_deps)):
+        _build_torch_shim()
     if verbose:
         print("built", LIB, "and", TORCH_LIB)
     return LIB
 
 
 if __name__ == "__main__":
-    build(verbose=True)
+    build(verbose=True, incremental="--incremental" in sys.argv[1:])
     sys.exit(0)

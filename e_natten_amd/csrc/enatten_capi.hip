@@ -136,6 +136,34 @@ size_t enatten2d_bwd_workspace_bytes(int B, int heads, int H, int W) {
     return (size_t)B * heads * H * W * 2 * sizeof(float);
 }
 
+// Shared body of the two backward entry points: `workspace` holds two float32 per query.
+static int bwd2d(const char *fn, const void *q, const void *k, const void *v, const void *o,
+                 const void *d_o, const float *lse, void *dq, void *dk, void *dv,
+                 float *workspace, int B, int heads, int H, int W, int D, int kernel_size,
+                 int dtype, const int64_t *q_strides, const int64_t *k_strides,
+                 const int64_t *v_strides, const int64_t *o_strides, const int64_t *do_strides,
+                 float scale, void *stream) {
+    BwdArgs a;
+    int rc;
+    if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
+    if ((rc = make_view(fn, "k", k, k_strides, heads, H, W, D, &a.k))) return rc;
+    if ((rc = make_view(fn, "v", v, v_strides, heads, H, W, D, &a.v))) return rc;
+    if ((rc = make_view(fn, "o", o, o_strides, heads, H, W, D, &a.o))) return rc;
+    if ((rc = make_view(fn, "d_o", d_o, do_strides, heads, H, W, D, &a.d_o))) return rc;
+    if (!lse || !dq || !dk || !dv) {
+        set_error("%s: lse, dq, dk and dv must all be non-NULL", fn);
+        return ENATTEN_EINVAL;
+    }
+    a.lse = lse;
+    a.dq = dq; a.dk = dk; a.dv = dv;
+    a.delta = workspace;
+    a.zinv = a.delta + (size_t)B * heads * H * W;
+    a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (use_mfma(D, kernel_size, dtype)) return launch_bwd_mfma(a, dtype, g_path.load(), st);
+    return launch_bwd_simt(a, dtype, st);
+}
+
 int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,
                   const float *lse, void *dq, void *dk, void *dv, void *workspace, int B,
                   int heads, int H, int W, int D, int kernel_size, int dtype,
@@ -143,26 +171,70 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o, co
                   const int64_t *o_strides, const int64_t *do_strides, float scale,
                   void *stream) {
     const char *fn = "enatten2d_bwd";
-    int rc = check_shape(fn, B, heads, H, W, D, kernel_size, dtype);
+    const int rc = check_shape(fn, B, heads, H, W, D, kernel_size, dtype);
     if (rc) return rc;
-    BwdArgs a;
-    if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
-    if ((rc = make_view(fn, "k", k, k_strides, heads, H, W, D, &a.k))) return rc;
-    if ((rc = make_view(fn, "v", v, v_strides, heads, H, W, D, &a.v))) return rc;
-    if ((rc = make_view(fn, "o", o, o_strides, heads, H, W, D, &a.o))) return rc;
-    if ((rc = make_view(fn, "d_o", d_o, do_strides, heads, H, W, D, &a.d_o))) return rc;
-    if (!lse || !dq || !dk || !dv || !workspace) {
-        set_error("%s: lse, dq, dk, dv and workspace must all be non-NULL", fn);
+    if (!workspace) {
+        set_error("%s: workspace is NULL", fn);
         return ENATTEN_EINVAL;
     }
-    a.lse = lse;
-    a.dq = dq; a.dk = dk; a.dv = dv;
-    a.delta = static_cast<float *>(workspace);
-    a.zinv = a.delta + (size_t)B * heads * H * W;
-    a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (use_mfma(D, kernel_size, dtype)) return launch_bwd_mfma(a, dtype, g_path.load(), st);
-    return launch_bwd_simt(a, dtype, st);
+    return bwd2d(fn, q, k, v, o, d_o, lse, dq, dk, dv, static_cast<float *>(workspace), B, heads,
+                 H, W, D, kernel_size, dtype, q_strides, k_strides, v_strides, o_strides,
+                 do_strides, scale, stream);
+}
+
+// ---- backward without a caller-provided workspace ---------------------------
+// The two float32 per query that the backward passes hand to each other live in a
+// device array of this library instead.  Every GPU holds its own copy of the array at
+// its own address; `scratch` below is only the host-side handle of the symbol, the
+// address on the current device comes from hipGetSymbolAddress, once per device.
+static __device__ __align__(256) float scratch[2 * (size_t)ENATTEN_STATIC_BWD_MAX_QUERIES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<float *> g_scratch_ptr[kMaxDevices];
+
+int scratch_of_current_device(const char *fn, float **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("%s: no current HIP device (or a device number beyond %d)", fn, kMaxDevices - 1);
+        return ENATTEN_ELAUNCH;
+    }
+    float *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        // two threads may both ask; they get the same answer
+        const hipError_t e = hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            set_error("%s: hipGetSymbolAddress(scratch) failed: %s", fn, hipGetErrorString(e));
+            return ENATTEN_ELAUNCH;
+        }
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return ENATTEN_OK;
+}
+}  // namespace
+
+int enatten2d_bwd_static(const void *q, const void *k, const void *v, const void *o,
+                         const void *d_o, const float *lse, void *dq, void *dk, void *dv, int B,
+                         int heads, int H, int W, int D, int kernel_size, int dtype,
+                         const int64_t *q_strides, const int64_t *k_strides,
+                         const int64_t *v_strides, const int64_t *o_strides,
+                         const int64_t *do_strides, float scale, void *stream) {
+    const char *fn = "enatten2d_bwd_static";
+    int rc = check_shape(fn, B, heads, H, W, D, kernel_size, dtype);
+    if (rc) return rc;
+    if ((int64_t)B * heads * H * W > (int64_t)ENATTEN_STATIC_BWD_MAX_QUERIES) {
+        set_error("%s: %lld queries exceed the %d that the built-in scratch holds; use "
+                  "enatten2d_bwd with a workspace", fn, (long long)B * heads * H * W,
+                  ENATTEN_STATIC_BWD_MAX_QUERIES);
+        return ENATTEN_EUNSUPPORTED;
+    }
+    float *ws = nullptr;
+    if ((rc = scratch_of_current_device(fn, &ws))) return rc;
+    // Nothing in the scratch has to start at zero: the first pass writes both values of
+    // every query before the second pass reads them.
+    return bwd2d(fn, q, k, v, o, d_o, lse, dq, dk, dv, ws, B, heads, H, W, D, kernel_size, dtype,
+                 q_strides, k_strides, v_strides, o_strides, do_strides, scale, stream);
 }
 
 static int view_1d(const char *fn, const char *name, const void *p, const int64_t *st, int N,

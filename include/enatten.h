@@ -115,6 +115,26 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o,
                   void *stream);
 
 /*
+ * enatten2d_bwd for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments and results as enatten2d_bwd without
+ * the workspace: the two float32 per query live in a device array that is part of
+ * this library (8 MiB on every GPU the library runs on, held until the process ends),
+ * so calls of at most ENATTEN_STATIC_BWD_MAX_QUERIES = B * heads * H * W queries are
+ * served and larger ones return ENATTEN_EUNSUPPORTED.  The call allocates and frees
+ * nothing.  The stream's device must be the current device.  All calls on one GPU
+ * share the one array: calls that may overlap there (different streams, different
+ * threads) race; order them.
+ */
+#define ENATTEN_STATIC_BWD_MAX_QUERIES (1 << 20)
+int enatten2d_bwd_static(const void *q, const void *k, const void *v, const void *o,
+                         const void *d_o, const float *lse, void *dq, void *dk, void *dv,
+                         int B, int heads, int H, int W, int D, int kernel_size, int dtype,
+                         const int64_t *q_strides, const int64_t *k_strides,
+                         const int64_t *v_strides, const int64_t *o_strides,
+                         const int64_t *do_strides, float scale, void *stream);
+
+/*
  * 1D neighborhood attention on [B, heads, T, D] tensors: query t attends the
  * kernel_size keys starting at clamp(t - kernel_size/2, 0, T - kernel_size).
  * Replace the launches of _attn_fwd_1d / _attn_bwd_1d in Natten1d
