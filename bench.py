@@ -5,9 +5,17 @@ and the C ABI) on the reference's benchmark shape (bench.py:14,39 of the
 reference: B=4, heads=4, head_dim=128, kernel_size=5) in bf16 at image side 128.
 Prints ONE JSON line.  `value` is useful TFLOP/s (14*k^2*d FLOP per query);
 `roofline` is the achieved algorithmic HBM bandwidth of the slowest kernel, from
-HIP events recorded around every kernel launch inside the timed region;
+HIP events recorded around kernel launches inside the timed region;
 `cpu_baseline` times the CPU restatement of the reference's algorithm on this
 machine's host cores on a bounded sample of the same workload.
+
+Cold and hot: the timed steps rotate over several sets of q, k, v, dO that together
+exceed twice the 256 MB memory-side cache, so every step finds its inputs in HBM
+(the reference's triton.testing.do_bench, its bench.py:28,59, flushes the cache
+between iterations for the same reason); `hot_ms_per_step` repeats one set.  The
+sweep rows say whether their working set fits that cache.  `unfused_gpu` times the
+unfused qk -> softmax -> av formulation in plain torch on the GPU, the comparator of
+the reference's benchmark (its bench.py:23,51-56 uses NATTEN's unfused ops).
 """
 from __future__ import annotations
 
@@ -23,8 +31,62 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
-MFMA_BF16_PEAK_TF = 2500.0   # dense bf16, published
+MFMA_PEAK_TF = {"bf16": 2500.0, "fp16": 2500.0}   # dense matrix-core peaks, published
+MALL_BYTES = 256 << 20       # memory-side (Infinity) cache
 KERNELS = ("fwd", "bwd_dq", "bwd_dkdv", "bwd_fused")
+
+
+def rotating_sets(shape, dtype, dev, tensors_per_set, seed=0, max_sets=600):
+    """Enough sets of `tensors_per_set` random tensors of `shape`, carved out of one
+    allocation, to exceed twice the memory-side cache (at least 3 sets).  Returns the
+    list of sets and whether their total really exceeds that bound."""
+    import torch
+    numel = 1
+    for x in shape:
+        numel *= x
+    esize = torch.empty((), dtype=dtype).element_size()
+    set_bytes = tensors_per_set * numel * esize
+    n = min(max_sets, max(3, -(-2 * MALL_BYTES // set_bytes) + 1))
+    g = torch.Generator(device=dev).manual_seed(seed)
+    big = torch.randn((n, tensors_per_set) + tuple(shape), generator=g, device=dev,
+                      dtype=torch.float32 if n * set_bytes < (8 << 30) else dtype).to(dtype)
+    return [tuple(big[i, j] for j in range(tensors_per_set)) for i in range(n)], \
+        n * set_bytes > 2 * MALL_BYTES
+
+
+def unfused_gpu(q, k, v, d_o, ks, iters=5):
+    """The unfused formulation on the GPU in plain torch, as NATTEN's qk / av ops
+    compute it (the reference's comparator, its bench.py:23 and :51-56): gather every
+    query's k*k keys, logits, softmax, gather the values, weighted sum; backward by
+    autograd.  Wall-clock per forward and per forward+backward."""
+    import torch
+    B, N, H, W, D = q.shape
+    dev = q.device
+    ar = lambda L: (torch.arange(L, device=dev) - ks // 2).clamp(0, L - ks)
+    rows = ar(H)[:, None] + torch.arange(ks, device=dev)[None, :]            # [H, k]
+    cols = ar(W)[:, None] + torch.arange(ks, device=dev)[None, :]            # [W, k]
+    idx = (rows[:, None, :, None] * W + cols[None, :, None, :]).reshape(H, W, ks * ks)
+
+    def fwd(q, k, v):
+        kg = k.flatten(2, 3)[:, :, idx]                                     # [B, N, H, W, k*k, D]
+        p = torch.softmax(torch.einsum("bnhwd,bnhwjd->bnhwj", q, kg).float(), dim=-1).to(q.dtype)
+        return torch.einsum("bnhwj,bnhwjd->bnhwd", p, v.flatten(2, 3)[:, :, idx])
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / iters
+
+    with torch.no_grad():
+        fwd_ms = timed(lambda: fwd(q, k, v))
+    qq, kk, vv = (t.detach().requires_grad_(True) for t in (q, k, v))
+    step_ms = timed(lambda: torch.autograd.grad(fwd(qq, kk, vv), (qq, kk, vv), d_o))
+    return {"fwd_ms": fwd_ms, "ms_per_step": step_ms,
+            "what": "torch gather + einsum + softmax on the GPU, %s" % str(q.dtype).replace("torch.", "")}
 
 
 def algorithmic_bytes(B, N, H, W, D, esize):
@@ -113,6 +175,8 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-sweep", action="store_true", help="skip the other image sides")
+    ap.add_argument("--no-unfused", action="store_true",
+                    help="skip the unfused qk -> softmax -> av comparator on the GPU")
     ap.add_argument("--simt", action="store_true", help="force the vector-ALU kernels")
     ap.add_argument("--fused-bwd", action="store_true",
                     help="force the fused backward kernel wherever it is built")
@@ -148,15 +212,19 @@ def main():
     shape = (B, N, S, S, D)
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(0)
-    q, k, v, d_o = (torch.randn(shape, generator=g).to(dtype).to(dev) for _ in range(4))
-    q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
+    sets, cold = rotating_sets(shape, dtype, dev, 4)
+    for st in sets:
+        for t in st[:3]:
+            t.requires_grad_(True)
+    q, k, v, d_o = sets[0]
 
-    def step():
+    def step(i=0):
+        q, k, v, d_o = sets[i % len(sets)]
         o = natten2d(q, k, v, ks)
         return torch.autograd.grad(o, (q, k, v), d_o)
 
-    for _ in range(args.warmup):
-        step()
+    for i in range(args.warmup):
+        step(i)
     torch.cuda.synchronize()
     # Per-kernel HIP events inside the timed region: every `period`-th launch of
     # each kernel is bracketed (a record costs ~3 us of queue time; timing all of
@@ -164,12 +232,21 @@ def main():
     period = max(1, args.steps // 10)
     lib.enatten_profile_enable(period)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    for i in range(args.steps):
+        step(i)
     host_s = time.perf_counter() - t0  # time to enqueue all steps
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     lib.enatten_profile_enable(0)
+    # the same steps on one set of inputs (whatever fits the caches stays there)
+    for _ in range(min(5, args.warmup)):
+        step(0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(0)
+    torch.cuda.synchronize()
+    hot_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
     if args.copy_calib:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
@@ -209,19 +286,27 @@ def main():
         "path_alg_bytes": alg["path"], "path_kernel_ms": kernel_ms,
         "path_GBps": alg["path"] / (kernel_ms * 1e-3) / 1e9,
         "path_frac": alg["path"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "mfma_frac_useful": useful / (kernel_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TF,
     }
+    path = kernel_path(D, ks, dtype)
+    if path == "mfma" and args.dtype in MFMA_PEAK_TF and not args.simt:
+        # useful FLOPs against the matrix-core peak of the dtype the kernels compute in
+        roofline["mfma_frac_useful"] = useful / (kernel_ms * 1e-3) / 1e12 / MFMA_PEAK_TF[args.dtype]
+    working_set = 8 * B * N * S * S * D * q.element_size()   # q, k, v, o, dO, dq, dk, dv
     out = {
-        "metric": "natten2d fwd+bwd useful TFLOP/s (B4 H4 d128 k5 bf16)",
+        "metric": "natten2d fwd+bwd useful TFLOP/s (B%d H%d d%d k%d %s)" % (B, N, D, ks, args.dtype),
         "value": useful / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "timing": "cold: %d input sets in rotation (%s twice the 256 MB memory-side cache)"
+                  % (len(sets), "more than" if cold else "LESS than"),
+        "hot_ms_per_step": hot_ms,
+        "working_set_fits_memory_side_cache": working_set <= MALL_BYTES,
         "host_enqueue_ms_per_step": host_s * 1e3 / args.steps,
         "kernel_event_sampling": "every %d-th launch" % period,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": "natten2d fwd+bwd B=%d heads=%d H=W=%d head_dim=%d kernel_size=%d"
                                % (B, N, S, D, ks),
-                   "kernel_path": kernel_path(D, ks, dtype), "queries": queries,
+                   "kernel_path": "simt" if args.simt else path, "queries": queries,
                    "useful_gflop": useful / 1e9},
         "roofline": roofline,
     }
@@ -230,42 +315,70 @@ def main():
         # only, under no_grad, sides 16..512; bench.py:34: forward+backward, sides
         # 16..256), wall-clock only, a few steps each.
         def wall_ms(fn, iters=20):
-            for _ in range(5):
-                fn()
+            for i in range(5):
+                fn(i)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            for _ in range(iters):
-                fn()
+            for i in range(iters):
+                fn(i)
             torch.cuda.synchronize()
             return (time.perf_counter() - t0) * 1e3 / iters
 
+        del sets
+        torch.cuda.empty_cache()
         sweep = []
+        esize = q.element_size()
         for side in (16, 32, 64, 128, 256, 512):
             shp = (B, N, side, side, D)
-            qs, ks_, vs = (torch.randn(shp, generator=g).to(dtype).to(dev) for _ in range(3))
+            ssets, scold = rotating_sets(shp, dtype, dev, 4 if side <= 256 else 3, seed=side)
             qn = B * N * side * side
             with torch.no_grad():
-                fwd_ms = wall_ms(lambda: natten2d(qs, ks_, vs, ks))
-            rec = {"side": side, "fwd_ms": fwd_ms,
-                   "fwd_frac_of_hbm_peak": (4 * qn * D * qs.element_size() + 4 * qn)
+                fwd_ms = wall_ms(lambda i: natten2d(*ssets[i % len(ssets)][:3], ks))
+                fwd_hot = wall_ms(lambda i: natten2d(*ssets[0][:3], ks))
+            rec = {"side": side, "fwd_ms": fwd_ms, "fwd_hot_ms": fwd_hot,
+                   "input_sets": len(ssets), "cold": scold,
+                   "fwd_working_set_fits_memory_side_cache": 4 * qn * D * esize <= MALL_BYTES,
+                   "fwd_frac_of_hbm_peak": (4 * qn * D * esize + 4 * qn)
                    / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
             if side <= 256 and side != S:
-                gs = torch.randn(shp, generator=g).to(dtype).to(dev)
-                for t in (qs, ks_, vs):
-                    t.requires_grad_(True)
-                ms = wall_ms(lambda: torch.autograd.grad(natten2d(qs, ks_, vs, ks), (qs, ks_, vs), gs))
+                for st in ssets:
+                    for t in st[:3]:
+                        t.requires_grad_(True)
+
+                def fb(i, rotate=True):
+                    qs, ks_, vs, gs = ssets[i % len(ssets) if rotate else 0]
+                    return torch.autograd.grad(natten2d(qs, ks_, vs, ks), (qs, ks_, vs), gs)
+                ms = wall_ms(fb)
+                ms_hot = wall_ms(lambda i: fb(i, False))
                 fl = 14.0 * ks * ks * D * qn
-                by = 11 * qn * D * qs.element_size() + 8 * qn
-                rec.update({"ms_per_step": ms, "useful_tflops": fl / ms / 1e9,
-                            "path_frac_of_hbm_peak": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                            "mfma_frac_useful": fl / ms / 1e9 / MFMA_BF16_PEAK_TF})
-                del gs
+                by = 11 * qn * D * esize + 8 * qn
+                rec.update({"ms_per_step": ms, "hot_ms_per_step": ms_hot,
+                            "working_set_fits_memory_side_cache": 8 * qn * D * esize <= MALL_BYTES,
+                            "useful_tflops": fl / ms / 1e9,
+                            "path_frac_of_hbm_peak": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
             sweep.append(rec)
-            del qs, ks_, vs
+            del ssets
+            torch.cuda.empty_cache()
         out["sweep"] = sweep
+    if not args.no_unfused:
+        gq = torch.Generator(device=dev).manual_seed(1)
+        uq, uk, uv, ug = (torch.randn(shape, generator=gq, device=dev, dtype=torch.float32).to(dtype)
+                          for _ in range(4))
+        try:
+            out["unfused_gpu"] = unfused_gpu(uq, uk, uv, ug, ks)
+            out["unfused_gpu"]["speedup_fwd_bwd"] = out["unfused_gpu"]["ms_per_step"] / ms_step
+        except torch.cuda.OutOfMemoryError as e:
+            out["unfused_gpu"] = {"error": "out of memory: %s" % str(e)[:80]}
+        del uq, uk, uv, ug
+        torch.cuda.empty_cache()
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(shape, ks, dtype, useful)
-        out["cpu_baseline"]["gpu_speedup"] = out["cpu_baseline"]["ms"] / ms_step
+        cb = cpu_baseline(shape, ks, dtype, useful)
+        # against the loop port (the headline baseline) and, the conservative figures,
+        # against the vectorised torch oracle and the C/OpenMP oracle on all host threads
+        cb["gpu_speedup"] = cb["ms"] / ms_step
+        cb["gpu_speedup_vs_vectorised_gather"] = cb["vectorised_gather_ms"] / ms_step
+        cb["gpu_speedup_vs_c_openmp"] = cb["c_openmp_ms"] / ms_step
+        out["cpu_baseline"] = cb
     print(json.dumps(out))
 
 

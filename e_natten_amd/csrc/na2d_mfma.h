@@ -147,10 +147,56 @@ struct Geo {
     static constexpr int NKP = (NK + 31) / 32 * 32;
     static constexpr int MT = NKP / 16;           // 16-token MFMA row tiles
     static constexpr int KSTEPS = NKP / 32;       // reduction steps of the second product
-    static constexpr int PITCH = D + 8;           // LDS row pitch in elements (16 B pad)
+    // LDS layout.  A row holds the D channels of one pixel.  Two layouts are written
+    // down; SWZ picks one at compile time and every address goes through the helpers
+    // below, which fold to plain constants for the padded layout.
+    //  * padded (SWZ = false): rows D + 8 elements apart.  The rows of an MFMA operand
+    //    tile (one row per lane, the same 16-byte chunk of each) then start 4 banks
+    //    apart; a 16-byte operand read costs 12 LDS cycles against 8.3 for a conflict-free
+    //    one (measured on the token pattern of kernel_size 5).
+    //  * swizzled (SWZ = true): rows D elements apart, chunk c of row r kept at chunk
+    //    position c ^ key(r), where key(r) runs through all CPR values over the rows that
+    //    share one 256-byte line of the 64 banks and the lines after it.  Operand reads
+    //    are then conflict-free and LDS holds 6-20% more pixels, but every read address
+    //    needs an XOR with a per-lane value instead of a constant offset: at head_dim 128,
+    //    kernel_size 5 the forward, dQ and dK/dV kernels execute 27% more vector
+    //    instructions with it, LDS conflict cycles fall from 44-52% to 34-39% of the LDS
+    //    cycles, and the kernels get 3-5% SLOWER (they wait on memory and instruction
+    //    latency, not on LDS bandwidth, which is about a third used).  So it is off.
+    static constexpr bool SWZ = false;
+    static constexpr int PITCH = SWZ ? D : D + 8;  // LDS row pitch in elements
     static constexpr int ROWS = HR * HC + 1;      // + one all-zero row for padding tokens
     static constexpr int ZROW = HR * HC;
     static constexpr int CPR = D / 8;             // 16-byte chunks per row
+    static constexpr int RPL = 16 / CPR;          // rows per 256-byte line (1, 2 or 4)
+    static constexpr int LB = D == 128 ? 2 : D == 64 ? 1 : 0;  // log2(D / 32)
+    static __device__ __forceinline__ int key(int row) { return SWZ ? (row / RPL) & (CPR - 1) : 0; }
+    // element offset of chunk c of a row
+    static __device__ __forceinline__ int chunk_at(int row, int c) {
+        return row * PITCH + ((c ^ key(row)) << 3);
+    }
+    // A operand of the first products: lane group g reads chunk g + 4 * ds of its row for
+    // ds = 0 .. DS-1.  a_row gives the address for ds = 0 up to the XOR with the high part
+    // of the key, a_at the address for a given (compile-time) ds.
+    struct ARow { const short *p; int kh; };
+    static __device__ __forceinline__ ARow a_row(const short *lds, int row, int g) {
+        const int k = key(row);
+        return ARow{lds + row * PITCH + ((g ^ (k & 3)) << 3), k >> 2};
+    }
+    static __device__ __forceinline__ const short *a_at(const ARow &r, int ds) {
+        return r.p + ((ds ^ r.kh) << 5);
+    }
+    // A operand of the second products (transposing reads): lane n reads 4 elements at
+    // element (n & 3) * D/4 + mt * 4 of its row for mt = 0 .. DT-1, i.e. chunk
+    // ((n & 3) << LB) | (mt >> 1), half (mt & 1).
+    struct TRow { const short *p; int kl; };
+    static __device__ __forceinline__ TRow t_row(const short *lds, int row, int n) {
+        const int k = key(row);
+        return TRow{lds + row * PITCH + ((((n & 3) ^ (k >> LB)) << LB) << 3), k & ((1 << LB) - 1)};
+    }
+    static __device__ __forceinline__ const short *t_at(const TRow &r, int mt) {
+        return r.p + ((((mt >> 1) ^ r.kl) << 3) | ((mt & 1) << 2));
+    }
     static constexpr int DS = D / 32;             // reduction steps over channels
     static constexpr int DT = D / 16;             // 16-channel MFMA row tiles of the output
     static constexpr int NCH = HR * HC * CPR;     // 16-byte chunks per staged halo
@@ -262,7 +308,10 @@ __device__ __forceinline__ HaloPlan<D, KS, NW> make_plan() {
     static_assert(G::NT % G::CPR == 0, "a thread keeps one channel chunk");
     HaloPlan<D, KS, NW> pl;
     pl.ch8 = (threadIdx.x % G::CPR) * 8;
-    pl.lds0 = (threadIdx.x / G::CPR) * G::PITCH + pl.ch8;
+    // the rows of one thread's chunks are NT / CPR apart, a multiple of 16 * RPL, so they
+    // share one key and the chunk position is the same for all of them
+    static_assert((G::NT / G::CPR) % (16 * G::RPL) == 0, "one chunk position per thread");
+    pl.lds0 = G::chunk_at(threadIdx.x / G::CPR, threadIdx.x % G::CPR);
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
         int row = threadIdx.x / G::CPR + i * (G::NT / G::CPR);
@@ -297,7 +346,7 @@ __device__ __forceinline__ void halo_fetch(HaloRegs<D, KS, NW> &reg, const HaloP
         reg.v[i] = *reinterpret_cast<const u32x4 *>(base + off);
     }
 }
-// Registers -> LDS, channel-major with padded pitch.
+// Registers -> LDS, one row of D channels per pixel, chunks permuted (Geo::key).
 template <int D, int KS, int NW = 4>
 __device__ __forceinline__ void halo_commit(short *lds, const HaloPlan<D, KS, NW> &pl,
                                    const HaloRegs<D, KS, NW> &reg) {
@@ -345,8 +394,8 @@ __device__ __forceinline__ void halo_commit_rows(short *lds, const HaloPlan<D, K
         if (pix < G::HR * G::HC && r < nrows) {
             int slot = rot + r;
             slot = slot >= G::HR ? slot - G::HR : slot;
-            *reinterpret_cast<u32x4 *>(lds + (slot * G::HC + (pl.rc[i] & 255)) * G::PITCH + pl.ch8) =
-                reg.v[i];
+            *reinterpret_cast<u32x4 *>(lds + G::chunk_at(slot * G::HC + (pl.rc[i] & 255),
+                                                          threadIdx.x % G::CPR)) = reg.v[i];
         }
     }
 }
@@ -356,7 +405,7 @@ template <int D, int KS, int NW = 4>
 __device__ __forceinline__ void zero_row(short *lds) {
     using G = Geo<D, KS, NW>;
     if (threadIdx.x < G::CPR)
-        *reinterpret_cast<uint4 *>(lds + G::ZROW * G::PITCH + threadIdx.x * 8) =
+        *reinterpret_cast<uint4 *>(lds + G::ZROW * G::PITCH + threadIdx.x * 8) =  // all zero: any order
             make_uint4(0, 0, 0, 0);
 }
 

@@ -115,12 +115,11 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
                 const int kk = mt * 16 + n;
-                const int row = trow(kk);
-                const short *kp = lds_k + row * G::PITCH + g * 8;
+                const typename G::ARow kp = G::a_row(lds_k, trow(kk), g);
                 f32x4 c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ds = 0; ds < G::DS; ds++)
-                    c = mfma16<BF>(*reinterpret_cast<const s16x8 *>(kp + ds * 32), qreg[ds], c);
+                    c = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(kp, ds)), qreg[ds], c);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int tk = mt * 16 + g * 4 + i;  // halo token of accumulator row g*4+i
@@ -152,17 +151,14 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
             for (int mt = 0; mt < G::DT; mt++) o[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < G::KSTEPS; ks++) {
-                const short *vp[2];
+                typename G::TRow vp[2];
 #pragma unroll
-                for (int h = 0; h < 2; h++) {
-                    const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
-                    const int row = trow(tk);
-                    vp[h] = lds_v + row * G::PITCH + (n & 3) * (D / 4);
-                }
+                for (int h = 0; h < 2; h++)
+                    vp[h] = G::t_row(lds_v, trow(ks * 32 + h * 16 + g * 4 + (n >> 2)), n);
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++)
                     o[mt] = mfma16<BF>(
-                        cat(lds_read_tr(vp[0] + mt * 4), lds_read_tr(vp[1] + mt * 4)), pb[ks],
+                        cat(lds_read_tr(G::t_at(vp[0], mt)), lds_read_tr(G::t_at(vp[1], mt))), pb[ks],
                         o[mt]);
             }
 
@@ -288,13 +284,12 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
             for (int mt = 0; mt < G::MT; mt++) {
                 const int kk = mt * 16 + n;
                 const int row = trow(kk);
-                const short *kp = lds_k + row * G::PITCH + g * 8;
-                const short *vp = lds_v + row * G::PITCH + g * 8;
+                const typename G::ARow kp = G::a_row(lds_k, row, g), vp = G::a_row(lds_v, row, g);
                 f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ds = 0; ds < G::DS; ds++) {
-                    cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(kp + ds * 32), qreg[ds], cs);
-                    cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(vp + ds * 32), greg[ds], cp);
+                    cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(kp, ds)), qreg[ds], cs);
+                    cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(vp, ds)), greg[ds], cp);
                 }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -315,12 +310,11 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
                 if constexpr (kKeepDp) {
                     cp = dp[mt];
                 } else {
-                    const int row = trow(mt * 16 + n);
-                    const short *vp = lds_v + row * G::PITCH + g * 8;
+                    const typename G::ARow vp = G::a_row(lds_v, trow(mt * 16 + n), g);
                     cp = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int ds = 0; ds < G::DS; ds++)
-                        cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(vp + ds * 32), greg[ds], cp);
+                        cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(vp, ds)), greg[ds], cp);
                 }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -334,17 +328,14 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
             for (int mt = 0; mt < G::DT; mt++) dq[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < G::KSTEPS; ks++) {
-                const short *kp[2];
+                typename G::TRow kp[2];
 #pragma unroll
-                for (int h = 0; h < 2; h++) {
-                    const int tk = ks * 32 + h * 16 + g * 4 + (n >> 2);
-                    const int row = trow(tk);
-                    kp[h] = lds_k + row * G::PITCH + (n & 3) * (D / 4);
-                }
+                for (int h = 0; h < 2; h++)
+                    kp[h] = G::t_row(lds_k, trow(ks * 32 + h * 16 + g * 4 + (n >> 2)), n);
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++)
                     dq[mt] = mfma16<BF>(
-                        cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)), dsb[ks],
+                        cat(lds_read_tr(G::t_at(kp[0], mt)), lds_read_tr(G::t_at(kp[1], mt))), dsb[ks],
                         dq[mt]);
             }
 
@@ -523,13 +514,12 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
             for (int m2 = 0; m2 < 2; m2++) {
                 const int mt = ks * 2 + m2;
                 const int row = row_of(mt * 16 + n);
-                const short *qp = lds_q + row * G::PITCH + g * 8;
-                const short *gp = lds_g + row * G::PITCH + g * 8;
+                const typename G::ARow qp = G::a_row(lds_q, row, g), gp = G::a_row(lds_g, row, g);
                 f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ds = 0; ds < G::DS; ds++) {
-                    cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32), kreg[ds], cs);
-                    cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32), vreg[ds], cp);
+                    cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(qp, ds)), kreg[ds], cs);
+                    cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(gp, ds)), vreg[ds], cp);
                 }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -543,18 +533,18 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
                     dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
                 }
             }
-            const short *qt[2], *gt[2];
+            typename G::TRow qt[2], gt[2];
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 const int row = row_of(ks * 32 + h * 16 + g * 4 + (n >> 2));
-                qt[h] = lds_q + row * G::PITCH + (n & 3) * (D / 4);
-                gt[h] = lds_g + row * G::PITCH + (n & 3) * (D / 4);
+                qt[h] = G::t_row(lds_q, row, n);
+                gt[h] = G::t_row(lds_g, row, n);
             }
 #pragma unroll
             for (int mt = 0; mt < G::DT; mt++) {
-                dv[mt] = mfma16<BF>(cat(lds_read_tr(gt[0] + mt * 4), lds_read_tr(gt[1] + mt * 4)),
+                dv[mt] = mfma16<BF>(cat(lds_read_tr(G::t_at(gt[0], mt)), lds_read_tr(G::t_at(gt[1], mt))),
                                     pb, dv[mt]);
-                dk[mt] = mfma16<BF>(cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)),
+                dk[mt] = mfma16<BF>(cat(lds_read_tr(G::t_at(qt[0], mt)), lds_read_tr(G::t_at(qt[1], mt))),
                                     dsb, dk[mt]);
             }
         }
@@ -695,13 +685,12 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 #pragma unroll
                 for (int m2 = 0; m2 < 2; m2++) {
                     const int row = row_of(q0 + m2 * 16 + n);
-                    const short *qp = lds_q + row * G::PITCH + g * 8;
-                    const short *gp = lds_g + row * G::PITCH + g * 8;
+                    const typename G::ARow qp = G::a_row(lds_q, row, g), gp = G::a_row(lds_g, row, g);
                     f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int ds = 0; ds < G::DS; ds++) {
-                        cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32), kreg[ds], cs);
-                        cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32), vreg[ds], cp);
+                        cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(qp, ds)), kreg[ds], cs);
+                        cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(gp, ds)), vreg[ds], cp);
                     }
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
@@ -719,19 +708,19 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
                         dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
                     }
                 }
-                const short *qt[2], *gt[2];
+                typename G::TRow qt[2], gt[2];
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
                     const int row = row_of(q0 + h * 16 + g * 4 + (n >> 2));
-                    qt[h] = lds_q + row * G::PITCH + (n & 3) * (D / 4);
-                    gt[h] = lds_g + row * G::PITCH + (n & 3) * (D / 4);
+                    qt[h] = G::t_row(lds_q, row, n);
+                    gt[h] = G::t_row(lds_g, row, n);
                 }
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++) {
                     dv[mt] = mfma16<BF>(
-                        cat(lds_read_tr(gt[0] + mt * 4), lds_read_tr(gt[1] + mt * 4)), pb, dv[mt]);
+                        cat(lds_read_tr(G::t_at(gt[0], mt)), lds_read_tr(G::t_at(gt[1], mt))), pb, dv[mt]);
                     dk[mt] = mfma16<BF>(
-                        cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)), dsb, dk[mt]);
+                        cat(lds_read_tr(G::t_at(qt[0], mt)), lds_read_tr(G::t_at(qt[1], mt))), dsb, dk[mt]);
                 }
             }
         }

@@ -248,7 +248,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
             const int pix = step_pixel(i, nr, role);
             if (pix >= 0) {
                 const int row = lds_row(pix / G::HC, pix % G::HC);
-                const int e = row * G::PITCH + ch8_of();
+                const int e = G::chunk_at(row, stid % G::CPR);
                 *reinterpret_cast<u32x4 *>(lds_q + e) = qst.v[i];
                 *reinterpret_cast<u32x4 *>(lds_g + e) = gst.v[i];
                 *reinterpret_cast<u32x4 *>(lds_k + e) = kst.v[i];
@@ -357,10 +357,13 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
             const int dr = win_start(py, s.H, KS) - sy0, dc = win_start(px, s.W, KS) - sx0;
             set_slots(orow);
             s16x8 qreg[G::DS], greg[G::DS];
+            {
+                const typename G::ARow qp = G::a_row(lds_q, prow, g), gp = G::a_row(lds_g, prow, g);
 #pragma unroll
-            for (int ds = 0; ds < G::DS; ds++) {
-                qreg[ds] = *reinterpret_cast<const s16x8 *>(lds_q + prow * G::PITCH + ds * 32 + g * 8);
-                greg[ds] = *reinterpret_cast<const s16x8 *>(lds_g + prow * G::PITCH + ds * 32 + g * 8);
+                for (int ds = 0; ds < G::DS; ds++) {
+                    qreg[ds] = *reinterpret_cast<const s16x8 *>(G::a_at(qp, ds));
+                    greg[ds] = *reinterpret_cast<const s16x8 *>(G::a_at(gp, ds));
+                }
             }
             const float2 mine = lds_stat[prow];
             const float lse2 = mine.x, delta = mine.y;
@@ -369,13 +372,12 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
             for (int mt = 0; mt < G::MT; mt++) {
                 if (mt < 4) issue(mt);
                 const int row = tok_row(2 * mt, n >> 3, ocol + (n & 7));
-                const short *kp = lds_k + row * G::PITCH + g * 8;
-                const short *vp = lds_v + row * G::PITCH + g * 8;
+                const typename G::ARow kp = G::a_row(lds_k, row, g), vp = G::a_row(lds_v, row, g);
                 f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ds = 0; ds < G::DS; ds++) {
-                    cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(kp + ds * 32), qreg[ds], cs);
-                    cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(vp + ds * 32), greg[ds], cp);
+                    cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(kp, ds)), qreg[ds], cs);
+                    cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(vp, ds)), greg[ds], cp);
                 }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -392,16 +394,14 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
             for (int mt = 0; mt < G::DT; mt++) dq[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < G::KSTEPS; ks++) {
-                const short *kp[2];
+                typename G::TRow kp[2];
 #pragma unroll
                 for (int h = 0; h < 2; h++)
-                    kp[h] = lds_k +
-                            tok_row(4 * ks + 2 * h, g >> 1, ocol + 4 * (g & 1) + (n >> 2)) * G::PITCH +
-                            (n & 3) * (D / 4);
+                    kp[h] = G::t_row(lds_k, tok_row(4 * ks + 2 * h, g >> 1, ocol + 4 * (g & 1) + (n >> 2)), n);
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++)
                     dq[mt] = mfma16<BF>(
-                        cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)), dsb[ks],
+                        cat(lds_read_tr(G::t_at(kp[0], mt)), lds_read_tr(G::t_at(kp[1], mt))), dsb[ks],
                         dq[mt]);
             }
             store_token<BF, D>(static_cast<short *>(a.dq) + out_token() * D, g, dq, s.scale, true);
@@ -419,22 +419,24 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 s16x8 pb[G::KSTEPS], dsb[G::KSTEPS];
                 {
                     s16x8 kreg[G::DS], vreg[G::DS];
+                    {
+                        const typename G::ARow kp = G::a_row(lds_k, prow, g), vp = G::a_row(lds_v, prow, g);
 #pragma unroll
-                    for (int ds = 0; ds < G::DS; ds++) {
-                        kreg[ds] = *reinterpret_cast<const s16x8 *>(lds_k + prow * G::PITCH + ds * 32 + g * 8);
-                        vreg[ds] = *reinterpret_cast<const s16x8 *>(lds_v + prow * G::PITCH + ds * 32 + g * 8);
+                        for (int ds = 0; ds < G::DS; ds++) {
+                            kreg[ds] = *reinterpret_cast<const s16x8 *>(G::a_at(kp, ds));
+                            vreg[ds] = *reinterpret_cast<const s16x8 *>(G::a_at(vp, ds));
+                        }
                     }
 #pragma unroll
                     for (int mt = 0; mt < G::MT; mt++) {
                         if (mt < 4) issue(mt);
                         const int row = tok_row(2 * mt, n >> 3, ocol + (n & 7));
-                        const short *qp = lds_q + row * G::PITCH + g * 8;
-                        const short *gp = lds_g + row * G::PITCH + g * 8;
+                        const typename G::ARow qp = G::a_row(lds_q, row, g), gp = G::a_row(lds_g, row, g);
                         f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int ds = 0; ds < G::DS; ds++) {
-                            cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32), kreg[ds], cs);
-                            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32), vreg[ds], cp);
+                            cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(qp, ds)), kreg[ds], cs);
+                            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(gp, ds)), vreg[ds], cp);
                         }
                         // queries of accumulator rows g*4 .. g*4+3: halo row 2*mt + g/2,
                         // columns 4*(g%2) .. +3, i.e. four consecutive LDS rows
@@ -459,17 +461,14 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                     for (int mt = 0; mt < G::DT; mt++) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int ks = 0; ks < G::KSTEPS; ks++) {
-                        const short *xt[2];
+                        typename G::TRow xt[2];
 #pragma unroll
                         for (int h = 0; h < 2; h++)
-                            xt[h] = lds_x +
-                                    tok_row(4 * ks + 2 * h, g >> 1, ocol + 4 * (g & 1) + (n >> 2)) *
-                                        G::PITCH +
-                                    (n & 3) * (D / 4);
+                            xt[h] = G::t_row(lds_x, tok_row(4 * ks + 2 * h, g >> 1, ocol + 4 * (g & 1) + (n >> 2)), n);
 #pragma unroll
                         for (int mt = 0; mt < G::DT; mt++)
                             acc[mt] = mfma16<BF>(
-                                cat(lds_read_tr(xt[0] + mt * 4), lds_read_tr(xt[1] + mt * 4)), b[ks],
+                                cat(lds_read_tr(G::t_at(xt[0], mt)), lds_read_tr(G::t_at(xt[1], mt))), b[ks],
                                 acc[mt]);
                     }
                     store_token<BF, D>(static_cast<short *>(out) + tok * D, g, acc, mul, true);
@@ -513,7 +512,8 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 // this lane's key and value rows are read from LDS where they are used
                 // (the registers do not hold them beside the two accumulators and the
                 // next tile's rows)
-                int kvoff = prow * G::PITCH + g * 8;
+                const int pkey = G::key(prow), kvh = pkey >> 2;
+                int kvoff = prow * G::PITCH + ((g ^ (pkey & 3)) << 3);
                 f32x4 dk[G::DT], dv[G::DT];
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++) {
@@ -534,15 +534,16 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                     for (int m2 = 0; m2 < 2; m2++) {
                         const int mt = ks * 2 + m2;
                         const int row = row_of(mt * 16 + n);
-                        const short *qp = lds_q + row * G::PITCH + g * 8;
-                        const short *gp = lds_g + row * G::PITCH + g * 8;
+                        const typename G::ARow qp = G::a_row(lds_q, row, g), gp = G::a_row(lds_g, row, g);
                         f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int ds = 0; ds < G::DS; ds++) {
-                            cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32),
-                                        *reinterpret_cast<const s16x8 *>(krow + ds * 32), cs);
-                            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32),
-                                            *reinterpret_cast<const s16x8 *>(vrow + ds * 32), cp);
+                            // the same logical chunk g + 4 * ds of the query row and of this
+                            // lane's key row, each where its own row keeps it
+                            cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(qp, ds)),
+                                        *reinterpret_cast<const s16x8 *>(krow + ((ds ^ kvh) << 5)), cs);
+                            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(gp, ds)),
+                                            *reinterpret_cast<const s16x8 *>(vrow + ((ds ^ kvh) << 5)), cp);
                         }
 #pragma unroll
                         for (int i = 0; i < 4; i++) {
@@ -553,18 +554,18 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                             dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
                         }
                     }
-                    const short *qt[2], *gt[2];
+                    typename G::TRow qt[2], gt[2];
 #pragma unroll
                     for (int h = 0; h < 2; h++) {
                         const int row = row_of(ks * 32 + h * 16 + g * 4 + (n >> 2));
-                        qt[h] = lds_q + row * G::PITCH + (n & 3) * (D / 4);
-                        gt[h] = lds_g + row * G::PITCH + (n & 3) * (D / 4);
+                        qt[h] = G::t_row(lds_q, row, n);
+                        gt[h] = G::t_row(lds_g, row, n);
                     }
 #pragma unroll
                     for (int mt = 0; mt < G::DT; mt++) {
-                        dv[mt] = mfma16<BF>(cat(lds_read_tr(gt[0] + mt * 4), lds_read_tr(gt[1] + mt * 4)),
+                        dv[mt] = mfma16<BF>(cat(lds_read_tr(G::t_at(gt[0], mt)), lds_read_tr(G::t_at(gt[1], mt))),
                                             pb, dv[mt]);
-                        dk[mt] = mfma16<BF>(cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)),
+                        dk[mt] = mfma16<BF>(cat(lds_read_tr(G::t_at(qt[0], mt)), lds_read_tr(G::t_at(qt[1], mt))),
                                             dsb, dk[mt]);
                     }
                 }
