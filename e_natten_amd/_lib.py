@@ -27,7 +27,7 @@ SIGNATURES = {
     "enatten2d_kernel_path": (_i, [_i, _i, _i]),
     "enatten_set_path": (_i, [_i]),
     "enatten2d_fwd": (_i, [_vp] * 5 + [_i] * 7 + [_sp] * 4 + [ctypes.c_float, _vp]),
-    "enatten2d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 4),
+    "enatten2d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 7),
     "enatten2d_bwd": (_i, [_vp] * 10 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
     "enatten2d_bwd_static": (_i, [_vp] * 9 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
     "enatten1d_fwd": (_i, [_vp] * 5 + [_i] * 6 + [_sp] * 4 + [ctypes.c_float, _vp]),

@@ -86,6 +86,14 @@ int make_view(const char *fn, const char *name, const void *p, const int64_t *st
 bool use_mfma(int D, int ks, int dtype) {
     return g_path.load() != ENATTEN_PATH_SIMT && mfma_supported(D, ks, dtype);
 }
+bool use_mfma_f32(int D, int ks, int dtype) {
+    return g_path.load() != ENATTEN_PATH_SIMT && mfma_f32_supported(D, ks, dtype);
+}
+// float32 per query of backward workspace: two for the general and the 16-bit kernels
+// (delta and 1/Z), 2 * ks * ks for the float32 matrix-core kernels (P and dS)
+size_t ws_floats_per_query(int D, int ks, int dtype) {
+    return mfma_f32_supported(D, ks, dtype) ? mfma_f32_workspace_floats(ks) : 2;
+}
 
 }  // namespace
 }  // namespace enatten
@@ -102,7 +110,8 @@ const char *enatten_last_error(void) { return g_err; }
 int enatten2d_kernel_path(int D, int kernel_size, int dtype) {
     if (elem_size(dtype) == 0 || D < 1 || D > 1024 || kernel_size < 1 || kernel_size % 2 == 0)
         return ENATTEN_PATH_NONE;
-    return use_mfma(D, kernel_size, dtype) ? ENATTEN_PATH_MFMA : ENATTEN_PATH_SIMT;
+    return use_mfma(D, kernel_size, dtype) || use_mfma_f32(D, kernel_size, dtype) ? ENATTEN_PATH_MFMA
+                                                                                  : ENATTEN_PATH_SIMT;
 }
 
 int enatten_set_path(int path) {
@@ -128,18 +137,20 @@ int enatten2d_fwd(const void *q, const void *k, const void *v, void *o, float *l
     a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (use_mfma(D, kernel_size, dtype)) return launch_fwd_mfma(a, dtype, st);
+    if (use_mfma_f32(D, kernel_size, dtype)) return launch_fwd_mfma_f32(a, st);
     return launch_fwd_simt(a, dtype, st);
 }
 
-size_t enatten2d_bwd_workspace_bytes(int B, int heads, int H, int W) {
-    if (B < 1 || heads < 1 || H < 1 || W < 1) return 0;
-    return (size_t)B * heads * H * W * 2 * sizeof(float);
+size_t enatten2d_bwd_workspace_bytes(int B, int heads, int H, int W, int D, int kernel_size,
+                                     int dtype) {
+    if (B < 1 || heads < 1 || H < 1 || W < 1 || D < 1 || kernel_size < 1) return 0;
+    return (size_t)B * heads * H * W * ws_floats_per_query(D, kernel_size, dtype) * sizeof(float);
 }
 
 // Shared body of the two backward entry points: `workspace` holds two float32 per query.
 static int bwd2d(const char *fn, const void *q, const void *k, const void *v, const void *o,
                  const void *d_o, const float *lse, void *dq, void *dk, void *dv,
-                 float *workspace, int B, int heads, int H, int W, int D, int kernel_size,
+                 float *workspace, size_t ws_floats, int B, int heads, int H, int W, int D, int kernel_size,
                  int dtype, const int64_t *q_strides, const int64_t *k_strides,
                  const int64_t *v_strides, const int64_t *o_strides, const int64_t *do_strides,
                  float scale, void *stream) {
@@ -161,6 +172,10 @@ static int bwd2d(const char *fn, const void *q, const void *k, const void *v, co
     a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (use_mfma(D, kernel_size, dtype)) return launch_bwd_mfma(a, dtype, g_path.load(), st);
+    // the float32 matrix-core backward where the workspace at hand holds its P and dS
+    if (use_mfma_f32(D, kernel_size, dtype) &&
+        ws_floats >= (size_t)B * heads * H * W * mfma_f32_workspace_floats(kernel_size))
+        return launch_bwd_mfma_f32(a, st);
     return launch_bwd_simt(a, dtype, st);
 }
 
@@ -177,7 +192,9 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o, co
         set_error("%s: workspace is NULL", fn);
         return ENATTEN_EINVAL;
     }
-    return bwd2d(fn, q, k, v, o, d_o, lse, dq, dk, dv, static_cast<float *>(workspace), B, heads,
+    // the caller provides enatten2d_bwd_workspace_bytes() for this very call
+    return bwd2d(fn, q, k, v, o, d_o, lse, dq, dk, dv, static_cast<float *>(workspace),
+                 (size_t)B * heads * H * W * ws_floats_per_query(D, kernel_size, dtype), B, heads,
                  H, W, D, kernel_size, dtype, q_strides, k_strides, v_strides, o_strides,
                  do_strides, scale, stream);
 }
@@ -233,7 +250,8 @@ int enatten2d_bwd_static(const void *q, const void *k, const void *v, const void
     if ((rc = scratch_of_current_device(fn, &ws))) return rc;
     // Nothing in the scratch has to start at zero: the first pass writes both values of
     // every query before the second pass reads them.
-    return bwd2d(fn, q, k, v, o, d_o, lse, dq, dk, dv, ws, B, heads, H, W, D, kernel_size, dtype,
+    return bwd2d(fn, q, k, v, o, d_o, lse, dq, dk, dv, ws,
+                 (size_t)2 * ENATTEN_STATIC_BWD_MAX_QUERIES, B, heads, H, W, D, kernel_size, dtype,
                  q_strides, k_strides, v_strides, o_strides, do_strides, scale, stream);
 }
 
@@ -288,7 +306,8 @@ int enatten1d_fwd(const void *q, const void *k, const void *v, void *o, float *l
 }
 
 size_t enatten1d_bwd_workspace_bytes(int B, int heads, int T) {
-    return enatten2d_bwd_workspace_bytes(B, heads, 1, T);
+    if (B < 1 || heads < 1 || T < 1) return 0;
+    return (size_t)B * heads * T * 2 * sizeof(float);
 }
 
 int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,

@@ -79,6 +79,13 @@ struct ProfScope {
 int launch_fwd_simt(const FwdArgs &a, int dtype, hipStream_t st);
 int launch_bwd_simt(const BwdArgs &a, int dtype, hipStream_t st);
 
+// float32 matrix-core kernels (float64 logits): D in {32, 64, 128}, kernel_size 3 / 5 / 7.
+// Their backward keeps 2 * ks * ks float32 per query in the workspace (a.delta).
+bool mfma_f32_supported(int D, int ks, int dtype);
+size_t mfma_f32_workspace_floats(int ks);
+int launch_fwd_mfma_f32(const FwdArgs &a, hipStream_t st);
+int launch_bwd_mfma_f32(const BwdArgs &a, hipStream_t st);
+
 // matrix-core kernels: bf16 / f16, D in {32, 64, 128}, square odd window
 bool mfma_supported(int D, int ks, int dtype);
 int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st);

@@ -110,7 +110,7 @@ std::tuple<Tensor, Tensor, Tensor> na2d_bwd(const Tensor &q_, const Tensor &k_, 
     const int B = q.size(0), N = q.size(1), H = q.size(2), W = q.size(3), D = q.size(4);
     Tensor dq = at::empty({B, N, H, W, D}, q.options());
     Tensor dk = at::empty_like(dq), dv = at::empty_like(dq);
-    Tensor ws = at::empty({(int64_t)enatten2d_bwd_workspace_bytes(B, N, H, W)},
+    Tensor ws = at::empty({(int64_t)enatten2d_bwd_workspace_bytes(B, N, H, W, D, (int)ks, dtype_code(q))},
                           q.options().dtype(at::kByte));
     check_rc(enatten2d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(),
                            lse.data_ptr<float>(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),

@@ -116,8 +116,9 @@ def _bwd_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
     with torch.cuda.device(q.device):
         dq = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
         dk, dv = torch.empty_like(dq), torch.empty_like(dq)
-        ws = torch.empty(lib.enatten2d_bwd_workspace_bytes(B, N, H, W), dtype=torch.uint8,
-                         device=q.device)
+        ws = torch.empty(lib.enatten2d_bwd_workspace_bytes(B, N, H, W, D, kernel_size,
+                                                            _DTYPES[q.dtype]),
+                         dtype=torch.uint8, device=q.device)
         _check(lib.enatten2d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                  d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
                                  dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, kernel_size,

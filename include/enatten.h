@@ -88,9 +88,13 @@ int enatten2d_fwd(const void *q, const void *k, const void *v, void *o, float *l
                   void *stream);
 
 /*
- * Bytes of device scratch enatten2d_bwd needs (two float32 per query).
+ * Bytes of device scratch enatten2d_bwd needs for a call of this shape: two float32
+ * per query, or 2 * kernel_size^2 per query where the float32 matrix-core kernels
+ * serve the call (they hand the probabilities and their gradients from the dQ pass to
+ * the dK/dV pass through it).
  */
-size_t enatten2d_bwd_workspace_bytes(int B, int heads, int H, int W);
+size_t enatten2d_bwd_workspace_bytes(int B, int heads, int H, int W, int D, int kernel_size,
+                                     int dtype);
 
 /*
  * Backward of 2D neighborhood attention.
@@ -104,7 +108,8 @@ size_t enatten2d_bwd_workspace_bytes(int B, int heads, int H, int W);
  *               through o_strides / do_strides
  *   lse         as written by enatten2d_fwd with the same scale
  *   dq, dk, dv  [B, heads, H, W, D] dtype, contiguous, fully overwritten
- *   workspace   enatten2d_bwd_workspace_bytes() bytes of device memory
+ *   workspace   enatten2d_bwd_workspace_bytes() bytes of device memory for this call's
+ *               shape, kernel_size and dtype
  */
 int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o,
                   const void *d_o, const float *lse, void *dq, void *dk, void *dv,
@@ -121,7 +126,8 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o,
  * the workspace: the two float32 per query live in a device array that is part of
  * this library (8 MiB on every GPU the library runs on, held until the process ends),
  * so calls of at most ENATTEN_STATIC_BWD_MAX_QUERIES = B * heads * H * W queries are
- * served and larger ones return ENATTEN_EUNSUPPORTED.  The call allocates and frees
+ * served and larger ones return ENATTEN_EUNSUPPORTED.  (float32 calls whose matrix-core
+ * backward would need more of it than the array holds run on the general kernels.)  The call allocates and frees
  * nothing.  The stream's device must be the current device.  All calls on one GPU
  * share the one array: calls that may overlap there (different streams, different
  * threads) race; order them.

@@ -82,7 +82,7 @@ def run_capi(q, k, v, d_o, ks, scale=1.0):
     B, N, H, W, D = q.shape
     o, dq, dk, dv = (torch.full_like(qd, float("nan")) for _ in range(4))
     lse = torch.full((B, N, H, W), float("nan"), dtype=torch.float32, device=dev)
-    ws = torch.full((lib.enatten2d_bwd_workspace_bytes(B, N, H, W) // 4 + 1,), float("nan"),
+    ws = torch.full((lib.enatten2d_bwd_workspace_bytes(B, N, H, W, D, ks, code) // 4 + 1,), float("nan"),
                     dtype=torch.float32, device=dev)
     st = torch.cuda.current_stream().cuda_stream
     rc = lib.enatten2d_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(),

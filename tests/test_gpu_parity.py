@@ -252,7 +252,7 @@ def test_output_written_into_callers_layout(shape, ks, _lib):
     o_view, g_view = o_buf.permute(0, 3, 1, 2, 4), g_buf.permute(0, 3, 1, 2, 4)
     lse = torch.empty((B, N, H, W), dtype=torch.float32, device=dev)
     dq, dk, dv = (torch.full(shape, float("nan"), dtype=BF, device=dev) for _ in range(3))
-    ws = torch.empty(_lib.enatten2d_bwd_workspace_bytes(B, N, H, W), dtype=torch.uint8, device=dev)
+    ws = torch.empty(_lib.enatten2d_bwd_workspace_bytes(B, N, H, W, D, ks, L.BF16), dtype=torch.uint8, device=dev)
     st = torch.cuda.current_stream().cuda_stream
     so, sg = L.strides4(o_view), L.strides4(g_view)
     rc = _lib.enatten2d_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o_buf.data_ptr(),

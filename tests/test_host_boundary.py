@@ -52,13 +52,17 @@ def test_c_abi_validates_before_launch(lib):
     # more than 2^40 elements: refused as unsupported, before any pointer is looked at
     assert lib.enatten2d_fwd(None, 1, 1, 1, None, 1 << 12, 1 << 12, 1 << 12, 1 << 12, 1024, 3, 0,
                              None, None, None, None, 1.0, None) == 2
-    assert lib.enatten2d_bwd_workspace_bytes(2, 3, 4, 5) == 2 * 3 * 4 * 5 * 8
-    assert lib.enatten2d_bwd_workspace_bytes(0, 3, 4, 5) == 0
+    assert lib.enatten2d_bwd_workspace_bytes(2, 3, 4, 5, 64, 3, 1) == 2 * 3 * 4 * 5 * 8
+    assert lib.enatten2d_bwd_workspace_bytes(0, 3, 4, 5, 64, 3, 1) == 0
+    # the float32 matrix-core backward keeps P and dS of every window position
+    assert lib.enatten2d_bwd_workspace_bytes(2, 3, 8, 8, 128, 5, 0) == 2 * 3 * 8 * 8 * 2 * 25 * 4
+    assert lib.enatten2d_bwd_workspace_bytes(2, 3, 16, 16, 128, 9, 0) == 2 * 3 * 16 * 16 * 8
 
 
 def test_kernel_path_query(lib):
     from e_natten_amd import kernel_path
-    assert kernel_path(128, 5, torch.float32) == "simt"
+    assert kernel_path(128, 5, torch.float32) == "mfma"    # float32 matrix-core kernels
+    assert kernel_path(128, 9, torch.float32) == "simt"
     assert kernel_path(2, 3, torch.float32) == "simt"
     assert kernel_path(128, 4, torch.bfloat16) == "none"
     assert kernel_path(4096, 3, torch.bfloat16) == "none"

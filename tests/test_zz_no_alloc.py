@@ -22,7 +22,7 @@ def _both(lib, shape, dtype, ks, seed):
     rc = lib.enatten2d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
                            B, N, H, W, D, ks, code, None, None, None, None, 1.0, st)
     assert rc == 0, L.last_error()
-    ws = torch.empty(lib.enatten2d_bwd_workspace_bytes(B, N, H, W), dtype=torch.uint8, device=dev)
+    ws = torch.empty(lib.enatten2d_bwd_workspace_bytes(B, N, H, W, D, ks, code), dtype=torch.uint8, device=dev)
     ref = [torch.full_like(q, float("nan")) for _ in range(3)]
     got = [torch.full_like(q, float("nan")) for _ in range(3)]
     rc = lib.enatten2d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), g.data_ptr(),
