@@ -126,14 +126,17 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
     }
 }
 
-template <int D, int KS, int NW = 4>
+template <int D, int KS, int NW = 4, int SP = 1>
 struct Geo {
     // NW waves own 4x4 pixel blocks, two side by side: a tile of 2*NW x 8 pixels.
     // Four waves (8x8 pixels) everywhere, except that the forward of a configuration
     // whose halo leaves room for only one workgroup per CU can use eight (16x8
     // pixels) where that still fits: two waves per SIMD, and less halo per pixel.
     static constexpr int TH = 2 * NW, TW = 8;     // pixels per workgroup
-    static constexpr int NT = 64 * NW;            // threads per workgroup
+    // SP waves share each 4x4 block: they split its halo tokens between them and add
+    // their partial sums at the end (used where LDS admits one workgroup per CU, so
+    // that a SIMD still holds two waves)
+    static constexpr int NT = 64 * NW * SP;       // threads per workgroup
     static constexpr int HR = TH + KS - 1;        // halo of the workgroup tile
     static constexpr int HC = TW + KS - 1;
     static constexpr int SW = 4 + KS - 1;         // halo side of one wave's 4x4 block
@@ -163,7 +166,10 @@ struct Geo {
     //    instructions with it, LDS conflict cycles fall from 44-52% to 34-39% of the LDS
     //    cycles, and the kernels get 3-5% SLOWER (they wait on memory and instruction
     //    latency, not on LDS bandwidth, which is about a third used).  So it is off.
-    static constexpr bool SWZ = false;
+#ifndef ENATTEN_SWZ_EXPR
+#define ENATTEN_SWZ_EXPR false
+#endif
+    static constexpr bool SWZ = ENATTEN_SWZ_EXPR;
     static constexpr int PITCH = SWZ ? D : D + 8;  // LDS row pitch in elements
     static constexpr int ROWS = HR * HC + 1;      // + one all-zero row for padding tokens
     static constexpr int ZROW = HR * HC;
@@ -206,7 +212,7 @@ struct Geo {
         (size_t)2 * ROWS * PITCH * sizeof(short) + ROWS * 2 * sizeof(float);
     // waves per SIMD to budget registers for: one per workgroup that LDS admits
     // on a CU (a workgroup puts one wave on each of the four SIMDs), at most 2
-    static constexpr int WAVES = NW == 4 ? (2 * LDS_BYTES <= 160 * 1024 ? 2 : 1) : 2;
+    static constexpr int WAVES = NW == 4 && SP == 1 ? (2 * LDS_BYTES <= 160 * 1024 ? 2 : 1) : 2;
     // staged LDS row of wave token tk whose halo starts at (orow, ocol) of the
     // staged block; numbers that are no token read the all-zero row
     static __device__ __forceinline__ int token_row(int tk, int orow, int ocol) {
@@ -296,17 +302,17 @@ __device__ __forceinline__ Tile tile_of(int t, int tiles_r, int tiles_c, int N, 
 // Staging plan of one thread: which 16-byte chunks of a halo it moves.  Chunk i of
 // thread t is chunk number t + 256*i of the halo in (row, column, channel-chunk)
 // order.  The plan is the same for every tile, so it is computed once.
-template <int D, int KS, int NW = 4>
+template <int D, int KS, int NW = 4, int SP = 1>
 struct HaloPlan {
-    int rc[Geo<D, KS, NW>::NL];  // halo row << 8 | halo column of chunk i
+    int rc[Geo<D, KS, NW, SP>::NL];  // halo row << 8 | halo column of chunk i
     int ch8;                 // first channel of the thread's chunks
     int lds0;                // LDS element offset of chunk 0
 };
-template <int D, int KS, int NW = 4>
-__device__ __forceinline__ HaloPlan<D, KS, NW> make_plan() {
-    using G = Geo<D, KS, NW>;
+template <int D, int KS, int NW = 4, int SP = 1>
+__device__ __forceinline__ HaloPlan<D, KS, NW, SP> make_plan() {
+    using G = Geo<D, KS, NW, SP>;
     static_assert(G::NT % G::CPR == 0, "a thread keeps one channel chunk");
-    HaloPlan<D, KS, NW> pl;
+    HaloPlan<D, KS, NW, SP> pl;
     pl.ch8 = (threadIdx.x % G::CPR) * 8;
     // the rows of one thread's chunks are NT / CPR apart, a multiple of 16 * RPL, so they
     // share one key and the chunk position is the same for all of them
@@ -320,9 +326,9 @@ __device__ __forceinline__ HaloPlan<D, KS, NW> make_plan() {
     }
     return pl;
 }
-template <int D, int KS, int NW = 4>
+template <int D, int KS, int NW = 4, int SP = 1>
 struct HaloRegs {
-    u32x4 v[Geo<D, KS, NW>::NL];
+    u32x4 v[Geo<D, KS, NW, SP>::NL];
 };
 // Global -> registers: this thread's share of the halo with origin (hr0, hc0) of
 // one image.  Halo positions at or beyond (rlim, clim) are not needed by any
@@ -330,11 +336,11 @@ struct HaloRegs {
 // stay in bounds and branch-free (the values only ever meet zero probabilities).
 // Addresses are a uniform base plus a 32-bit per-lane byte offset formed with
 // 24-bit multiplies: strides are below 2^22 elements (checked on the host).
-template <int D, int KS, int NW = 4>
-__device__ __forceinline__ void halo_fetch(HaloRegs<D, KS, NW> &reg, const HaloPlan<D, KS, NW> &pl,
+template <int D, int KS, int NW = 4, int SP = 1>
+__device__ __forceinline__ void halo_fetch(HaloRegs<D, KS, NW, SP> &reg, const HaloPlan<D, KS, NW, SP> &pl,
                                   const short *img, int64_t sh, int64_t sw, int hr0, int hc0,
                                   int rlim, int clim) {
-    using G = Geo<D, KS, NW>;
+    using G = Geo<D, KS, NW, SP>;
     const char *base = reinterpret_cast<const char *>(img + hr0 * sh + hc0 * sw);
     const unsigned sh2 = (unsigned)sh * 2u, sw2 = (unsigned)sw * 2u;
     const int rmax = rlim - 1 - hr0, cmax = clim - 1 - hc0;
@@ -347,10 +353,10 @@ __device__ __forceinline__ void halo_fetch(HaloRegs<D, KS, NW> &reg, const HaloP
     }
 }
 // Registers -> LDS, one row of D channels per pixel, chunks permuted (Geo::key).
-template <int D, int KS, int NW = 4>
-__device__ __forceinline__ void halo_commit(short *lds, const HaloPlan<D, KS, NW> &pl,
-                                   const HaloRegs<D, KS, NW> &reg) {
-    using G = Geo<D, KS, NW>;
+template <int D, int KS, int NW = 4, int SP = 1>
+__device__ __forceinline__ void halo_commit(short *lds, const HaloPlan<D, KS, NW, SP> &pl,
+                                   const HaloRegs<D, KS, NW, SP> &reg) {
+    using G = Geo<D, KS, NW, SP>;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
         const int row = threadIdx.x / G::CPR + i * (G::NT / G::CPR);
@@ -362,11 +368,11 @@ __device__ __forceinline__ void halo_commit(short *lds, const HaloPlan<D, KS, NW
 // in row slot y % HR): move only the `nrows` image rows from y0 on, all HC columns
 // from hc0 on.  A tile that follows its upper neighbour thus loads only the rows
 // the neighbour's halo did not hold.
-template <int D, int KS, int NW = 4>
-__device__ __forceinline__ void halo_fetch_rows(HaloRegs<D, KS, NW> &reg, const HaloPlan<D, KS, NW> &pl,
+template <int D, int KS, int NW = 4, int SP = 1>
+__device__ __forceinline__ void halo_fetch_rows(HaloRegs<D, KS, NW, SP> &reg, const HaloPlan<D, KS, NW, SP> &pl,
                                                 const short *img, int64_t sh, int64_t sw, int y0,
                                                 int hc0, int nrows, int rlim, int clim) {
-    using G = Geo<D, KS, NW>;
+    using G = Geo<D, KS, NW, SP>;
     const int yb = min(y0, rlim - 1);
     const char *base = reinterpret_cast<const char *>(img + yb * sh + hc0 * sw);
     const unsigned sh2 = (unsigned)sh * 2u, sw2 = (unsigned)sw * 2u;
@@ -382,10 +388,10 @@ __device__ __forceinline__ void halo_fetch_rows(HaloRegs<D, KS, NW> &reg, const 
         }
     }
 }
-template <int D, int KS, int NW = 4>
-__device__ __forceinline__ void halo_commit_rows(short *lds, const HaloPlan<D, KS, NW> &pl,
-                                                 const HaloRegs<D, KS, NW> &reg, int y0, int nrows) {
-    using G = Geo<D, KS, NW>;
+template <int D, int KS, int NW = 4, int SP = 1>
+__device__ __forceinline__ void halo_commit_rows(short *lds, const HaloPlan<D, KS, NW, SP> &pl,
+                                                 const HaloRegs<D, KS, NW, SP> &reg, int y0, int nrows) {
+    using G = Geo<D, KS, NW, SP>;
     const int rot = y0 % G::HR;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
@@ -401,9 +407,9 @@ __device__ __forceinline__ void halo_commit_rows(short *lds, const HaloPlan<D, K
 }
 // The spare row stays zero for the whole kernel: padding tokens and tokens
 // outside a wave's halo read it, so they add exact zeros to the second product.
-template <int D, int KS, int NW = 4>
+template <int D, int KS, int NW = 4, int SP = 1>
 __device__ __forceinline__ void zero_row(short *lds) {
-    using G = Geo<D, KS, NW>;
+    using G = Geo<D, KS, NW, SP>;
     if (threadIdx.x < G::CPR)
         *reinterpret_cast<uint4 *>(lds + G::ZROW * G::PITCH + threadIdx.x * 8) =  // all zero: any order
             make_uint4(0, 0, 0, 0);

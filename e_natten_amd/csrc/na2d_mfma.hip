@@ -26,6 +26,8 @@
 // softmax, P.V); the log-sum-exp is kept for the backward.
 
 
+#include <type_traits>
+
 #include "na2d_mfma.h"
 
 namespace enatten {
@@ -276,7 +278,10 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
             // the largest halos it is not kept but formed a second time once delta
             // is known (measured faster there: the matrix cores are idle, the
             // registers are not).
-            constexpr bool kKeepDp = !(G::WAVES == 1 && G::MT >= 16);
+#ifndef ENATTEN_KEEPDP_EXPR
+#define ENATTEN_KEEPDP_EXPR !(G::WAVES == 1 && G::MT >= 16)
+#endif
+            constexpr bool kKeepDp = ENATTEN_KEEPDP_EXPR;
             f32x4 dp[kKeepDp ? G::MT : 1];
             s16x8 dsb[G::KSTEPS];
             float dpart = 0.f;
@@ -390,19 +395,21 @@ __device__ __forceinline__ bool next_block(KeyBlock &b) {
 // queries and keys exchanged: the staged block is the tile's (8+k-1)^2 halo of
 // queries, a wave's queries are the (4+k-1)^2 halo of its 4x4 keys at a fixed
 // place in it, and the mask depends on the lane only.
-template <bool BF, int D, int KS, bool ROLL>
+template <bool BF, int D, int KS, bool ROLL, int SP>
 __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, int ntiles, Runs rp,
                                            int block, int nblocks, short *lds_q, short *lds_g,
-                                           float2 *lds_stat) {
-    using G = Geo<D, KS>;
+                                           float2 *lds_stat, f32x4 *lds_red) {
+    using G = Geo<D, KS, 4, SP>;
     const Shape &s = a.s;
     Sched sc = ROLL ? make_runs(ntiles, block, nblocks, rp) : make_sched(ntiles, block, nblocks);
     if (sc.t >= sc.t_end) return;
-    zero_row<D, KS>(lds_q);
-    zero_row<D, KS>(lds_g);
+    zero_row<D, KS, 4, SP>(lds_q);
+    zero_row<D, KS, 4, SP>(lds_g);
     if (threadIdx.x == 0) lds_stat[G::ZROW] = make_float2(0.f, 0.f);
 
-    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    // wave = block of 4x4 keys (0..3) + 4 * (its part of the block's queries)
+    const int wave = (threadIdx.x >> 6) & 3, part = threadIdx.x >> 8;
+    const int l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
     const int orow = (wave >> 1) * 4, ocol = (wave & 1) * 4;
     int rot = 0;  // ROLL: (first image row of the staged block) % HR
@@ -413,8 +420,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         return ROLL ? inner_tile_cm(t, ts, s.N) : inner_tile(t, ts, s.N);
     };
 
-    const HaloPlan<D, KS> plan = make_plan<D, KS>();
-    HaloRegs<D, KS> qst, gst;
+    const HaloPlan<D, KS, 4, SP> plan = make_plan<D, KS, 4, SP>();
+    HaloRegs<D, KS, 4, SP> qst, gst;
     float2 sst[G::NST];
     // ROLL: rows [y0, y0 + nr) of the block are what LDS does not hold yet
     auto prefetch = [&](const Tile &tl, int y0, int nr) __attribute__((always_inline)) {
@@ -429,7 +436,7 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         }
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
-            const int id = min((int)threadIdx.x + i * 256, G::ZROW - 1);
+            const int id = min((int)threadIdx.x + i * G::NT, G::ZROW - 1);
             const int pr = id / G::HC, pc = id % G::HC;
             if (!ROLL || pr < nr) {
                 const int64_t qt = img_tok + (int64_t)((ROLL ? y0 : br) + pr) * s.W + bc + pc;
@@ -444,7 +451,7 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
             const int r0m = y0 % G::HR;
 #pragma unroll
             for (int i = 0; i < G::NST; i++) {
-                const int id = threadIdx.x + i * 256;
+                const int id = threadIdx.x + i * G::NT;
                 const int pr = id / G::HC, pc = id % G::HC;
                 if (id < G::ZROW && pr < nr) {
                     int slot = r0m + pr;
@@ -457,7 +464,7 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
             halo_commit<D, KS>(lds_g, plan, gst);
 #pragma unroll
             for (int i = 0; i < G::NST; i++) {
-                const int id = threadIdx.x + i * 256;
+                const int id = threadIdx.x + i * G::NT;
                 if (id < G::ZROW) lds_stat[id] = sst[i];
             }
         }
@@ -507,8 +514,13 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
             dk[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
             dv[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
+        // this wave's share of the reduction steps (all of them if SP == 1)
+        auto steps = [&](auto part_c) __attribute__((always_inline)) {
+        constexpr int CH = (G::KSTEPS + SP - 1) / SP;
+        constexpr int K0 = decltype(part_c)::value * CH;
+        constexpr int K1 = K0 + CH < G::KSTEPS ? K0 + CH : G::KSTEPS;
 #pragma unroll
-        for (int ks = 0; ks < G::KSTEPS; ks++) {
+        for (int ks = K0; ks < K1; ks++) {
             s16x8 pb, dsb;
 #pragma unroll
             for (int m2 = 0; m2 < 2; m2++) {
@@ -548,39 +560,74 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
                                     dsb, dk[mt]);
             }
         }
+        };
+        if constexpr (SP == 1) {
+            steps(std::integral_constant<int, 0>{});
+        } else {
+            static_assert(SP == 2, "two parts");
+            if (part == 0) steps(std::integral_constant<int, 0>{});
+            else steps(std::integral_constant<int, 1>{});
+        }
 
-        {
+        auto store = [&]() __attribute__((always_inline)) {
             const int kr = cur.r0 + orow + (n >> 2), kc = cur.c0 + ocol + (n & 3);
             const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + kr) * s.W + kc;
             store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
             store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
+        };
+        if constexpr (SP == 1) {
+            store();
+            if (!more) break;
+            load_keys(nxt);
+            __syncthreads();
+        } else {
+            // the second part hands its sums to the first through LDS; the first adds
+            // and stores them once the barrier that ends the tile has passed (the
+            // second part writes again only after the next tile's first barrier)
+            f32x4 *red = lds_red + wave * 64 + l;
+            if (part == 1) {
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++) {
+                    red[mt * 256] = dk[mt];
+                    red[(G::DT + mt) * 256] = dv[mt];
+                }
+            }
+            if (more) load_keys(nxt);
+            __syncthreads();
+            if (part == 0) {
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++) {
+                    dk[mt] += red[mt * 256];
+                    dv[mt] += red[(G::DT + mt) * 256];
+                }
+                store();
+            }
+            if (!more) break;
         }
-
-        if (!more) break;
-        load_keys(nxt);
-        __syncthreads();
         cur = nxt;
         sched_advance(sc, tn);
     }
 }
 
 // Frame tiles: the general case, walked block by block (see above).
-template <bool BF, int D, int KS>
+template <bool BF, int D, int KS, int SP>
 __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, int ntiles,
                                            int block, int nblocks, short *lds_q, short *lds_g,
-                                           float2 *lds_stat) {
-    using G = Geo<D, KS>;
+                                           float2 *lds_stat, f32x4 *lds_red) {
+    using G = Geo<D, KS, 4, SP>;
     const Shape &s = a.s;
     Sched sc = make_sched(ntiles, block, nblocks);
     if (sc.t >= sc.t_end) return;
-    zero_row<D, KS>(lds_q);
-    zero_row<D, KS>(lds_g);
+    zero_row<D, KS, 4, SP>(lds_q);
+    zero_row<D, KS, 4, SP>(lds_g);
 
-    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    // wave = block of 4x4 keys (0..3) + 4 * (its part of the block's queries)
+    const int wave = (threadIdx.x >> 6) & 3, part = threadIdx.x >> 8;
+    const int l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
 
-    const HaloPlan<D, KS> plan = make_plan<D, KS>();
-    HaloRegs<D, KS> qst, gst;
+    const HaloPlan<D, KS, 4, SP> plan = make_plan<D, KS, 4, SP>();
+    HaloRegs<D, KS, 4, SP> qst, gst;
     float2 sst[G::NST];
     // the wave's 4x4 keys of a tile: this lane's key pixel (clamped into the image)
     auto key_of = [&](const Tile &tl, int &kr, int &kc) __attribute__((always_inline)) {
@@ -593,7 +640,7 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
         halo_fetch<D, KS>(gst, plan, image<short>(a.d_o, b.tl), a.d_o.sh, a.d_o.sw, b.br, b.bc, b.qb, b.cb);
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
-            const int id = threadIdx.x + i * 256;
+            const int id = threadIdx.x + i * G::NT;
             const int r = min(b.br + id / G::HC, b.qb - 1), c = min(b.bc + id % G::HC, b.cb - 1);
             const int64_t qt = img_tok + (int64_t)r * s.W + c;
             sst[i] = make_float2(a.lse[qt] * kLog2e, a.delta[qt]);
@@ -629,10 +676,11 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 
     f32x4 dk[G::DT], dv[G::DT];
     KeyBlock cur = first_of(sc.t);
-    // The loads of a block are issued when the previous block's math is over; the
-    // other workgroup on the CU covers their latency.  (These tiles are the
-    // minority; keeping the loads in flight across the math would need registers
-    // that the two accumulators do not leave.)
+    // With one part per block (SP == 1) the loads of a block are issued when the previous
+    // block's math is over and the other workgroup on the CU covers their latency
+    // (keeping them in flight across the math would need registers that the two
+    // accumulators do not leave).  With two parts a thread stages half as much, and the
+    // next block's loads are in flight while this one is computed.
     stage(cur);
     load_keys(cur.tl);
     for (;;) {
@@ -640,7 +688,7 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
         halo_commit<D, KS>(lds_g, plan, gst);
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
-            const int id = threadIdx.x + i * 256;
+            const int id = threadIdx.x + i * G::NT;
             if (id < G::ZROW) lds_stat[id] = sst[i];
             else if (id == G::ZROW) lds_stat[id] = make_float2(0.f, 0.f);
         }
@@ -658,6 +706,9 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
         if (!more && cur.t + sc.step < sc.t_end) {
             nxt = first_of(cur.t + sc.step);
             more = true;
+        }
+        if constexpr (SP > 1) {
+            if (more) stage(nxt);
         }
         const int wr0 = cur.tl.r0 + (wave >> 1) * 4, wc0 = cur.tl.c0 + (wave & 1) * 4;
         const bool wave_on = wr0 < s.H && wc0 < s.W;
@@ -680,7 +731,7 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
                 const int row = (ra + dvd - cur.br) * G::HC + (cc + qi - dvd * wcols - cur.bc);
                 return qi < nq ? row : (int)G::ZROW;
             };
-            for (int q0 = 0; q0 < nq; q0 += 32) {
+            for (int q0 = part * 32; q0 < nq; q0 += 32 * SP) {
                 s16x8 pb, dsb;
 #pragma unroll
                 for (int m2 = 0; m2 < 2; m2++) {
@@ -726,17 +777,40 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
         }
 
         const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
-        if (cur.last) {
+        auto store = [&]() __attribute__((always_inline)) {
             const int64_t tok =
                 (((int64_t)cur.tl.bb * s.N + cur.tl.nn) * s.H + kr) * s.W + kc;
             store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, live);
             store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, live);
+        };
+        if constexpr (SP == 1) {
+            if (cur.last) store();
+            if (!more) break;
+            stage(nxt);
+            if (nxt.first) load_keys(nxt.tl);
+            __syncthreads();
+        } else {
+            // the second part's sums reach the first through LDS (see dkdv_inner)
+            f32x4 *red = lds_red + wave * 64 + l;
+            if (cur.last && part == 1) {
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++) {
+                    red[mt * 256] = dk[mt];
+                    red[(G::DT + mt) * 256] = dv[mt];
+                }
+            }
+            if (more && nxt.first) load_keys(nxt.tl);
+            __syncthreads();
+            if (cur.last && part == 0) {
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++) {
+                    dk[mt] += red[mt * 256];
+                    dv[mt] += red[(G::DT + mt) * 256];
+                }
+                store();
+            }
+            if (!more) break;
         }
-
-        if (!more) break;
-        stage(nxt);
-        if (nxt.first) load_keys(nxt.tl);
-        __syncthreads();
         cur = nxt;
     }
 }
@@ -744,19 +818,23 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 // One launch for the whole dK/dV pass: the first `inner_blocks` workgroups sweep
 // the inner tiles, the rest the frame tiles, so the two kinds of work overlap on
 // every CU and end together.
-template <bool BF, int D, int KS, bool ROLL>
-__global__ __launch_bounds__(256, (Geo<D, KS>::WAVES)) void bwd_dkdv_mfma(BwdArgs a, TileSet ts,
-                                                                        int n_inner, int n_frame,
-                                                                        int inner_blocks, Runs rp) {
-    using G = Geo<D, KS>;
+// SP = 2: eight waves, two per 4x4 block of keys (see Geo), for halos that leave LDS for
+// one workgroup per CU.
+template <bool BF, int D, int KS, bool ROLL, int SP = 1>
+__global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (Geo<D, KS, 4, SP>::WAVES)) void bwd_dkdv_mfma(
+    BwdArgs a, TileSet ts, int n_inner, int n_frame, int inner_blocks, Runs rp) {
+    using G = Geo<D, KS, 4, SP>;
     __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
     __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
+    // partial dK and dV of the second part of every block
+    __shared__ f32x4 lds_red[SP > 1 ? 2 * G::DT * 256 : 1];
     if ((int)blockIdx.x < inner_blocks)
-        dkdv_inner<BF, D, KS, ROLL>(a, ts, n_inner, rp, blockIdx.x, inner_blocks, lds_q, lds_g, lds_stat);
+        dkdv_inner<BF, D, KS, ROLL, SP>(a, ts, n_inner, rp, blockIdx.x, inner_blocks, lds_q, lds_g,
+                                        lds_stat, lds_red);
     else
-        dkdv_frame<BF, D, KS>(a, ts, n_frame, blockIdx.x - inner_blocks,
-                              gridDim.x - inner_blocks, lds_q, lds_g, lds_stat);
+        dkdv_frame<BF, D, KS, SP>(a, ts, n_frame, blockIdx.x - inner_blocks,
+                                  gridDim.x - inner_blocks, lds_q, lds_g, lds_stat, lds_red);
 }
 
 // ------------------------------------------------------------------ dispatch
@@ -790,7 +868,20 @@ constexpr bool kTallBuilt =
     D == 64 && KS >= 7 &&
     (size_t)2 * Geo<D, KS, 8>::ROWS * Geo<D, KS, 8>::PITCH * sizeof(short) <= 160 * 1024;
 template <int D, int KS>
-constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= 11;
+#ifndef ENATTEN_TALLDQ_MAXK
+#define ENATTEN_TALLDQ_MAXK 11
+#endif
+constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= ENATTEN_TALLDQ_MAXK;
+
+// The dK/dV pass with two waves per 4x4 block of keys, each on half of the block's
+// queries (Geo's SP): where the staged queries leave LDS for one workgroup per CU, a
+// SIMD then still holds two waves.  Built for head_dim 64 (the partial sums of the
+// second wave pass through 32 KB of LDS there).
+#ifndef ENATTEN_DKDV_SPLIT_EXPR
+#define ENATTEN_DKDV_SPLIT_EXPR (D == 64 && Geo<D, KS>::WAVES == 1 ? 2 : 1)
+#endif
+template <int D, int KS>
+constexpr int kDkdvSplit = ENATTEN_DKDV_SPLIT_EXPR;
 
 template <bool BF, int D, int KS>
 int fwd_launch(const FwdArgs &a, hipStream_t st) {
@@ -885,8 +976,9 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             // Share the resident workgroups in proportion to the work.  Measured cost
             // of a frame tile in inner tiles: about 2 when the inner tiles are bound
             // by arithmetic (d <= 64), about 1.15 when they are bound by HBM (d = 128).
+            constexpr int SP = kDkdvSplit<D, KS>, NT = Geo<D, KS, 4, SP>::NT;
             const double cost = D >= 128 ? 1.15 : 2.0;
-            const int grid = persistent_grid<bwd_dkdv_mfma<BF, D, KS, false>>(nb);
+            const int grid = persistent_grid<bwd_dkdv_mfma<BF, D, KS, false, SP>>(nb, NT);
             int inner_blocks = 0;
             if (n_frame == 0) {
                 inner_blocks = grid;
@@ -899,11 +991,11 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             }
             ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
             if (inner_blocks > 0 && roll_pays<D>(n_inner, inner_blocks))
-                hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, kRollBuilt<D>>), dim3(grid), dim3(256),
+                hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, kRollBuilt<D>, SP>), dim3(grid), dim3(NT),
                                    0, st, a, ts, (int)n_inner, (int)n_frame, inner_blocks,
                                    plan_runs(n_inner, inner_blocks, ts.ni_r));
             else
-                hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, false>), dim3(grid), dim3(256), 0, st,
+                hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, false, SP>), dim3(grid), dim3(NT), 0, st,
                                    a, ts, (int)n_inner, (int)n_frame, inner_blocks, Runs{0, 0});
         }
         return check_launch("enatten2d_bwd");

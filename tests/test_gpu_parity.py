@@ -135,6 +135,8 @@ def test_config5_backbone_stages(heads, side, path):
     ((1, 2, 30, 31, 64), 9, BF),
     ((1, 1, 26, 27, 32), 11, BF),
     ((1, 1, 13, 13, 64), 13, BF),
+    ((1, 2, 37, 29, 64), 13, BF),    # two waves per block of keys in the dK/dV pass, ragged sides
+    ((2, 1, 43, 52, 64), 11, F16),
     ((2, 2, 12, 12, 32), 1, BF),     # k = 1: O == V
     ((1, 2, 20, 18, 64), 5, F16),
     ((1, 2, 20, 18, 128), 7, F16),
