@@ -26,8 +26,6 @@
 // softmax, P.V); the log-sum-exp is kept for the backward.
 
 
-#include <type_traits>
-
 #include "na2d_mfma.h"
 
 namespace enatten {
@@ -395,7 +393,7 @@ __device__ __forceinline__ bool next_block(KeyBlock &b) {
 // queries and keys exchanged: the staged block is the tile's (8+k-1)^2 halo of
 // queries, a wave's queries are the (4+k-1)^2 halo of its 4x4 keys at a fixed
 // place in it, and the mask depends on the lane only.
-template <bool BF, int D, int KS, bool ROLL, int SP>
+template <bool BF, int D, int KS, bool ROLL, int SP, int PART>
 __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, int ntiles, Runs rp,
                                            int block, int nblocks, short *lds_q, short *lds_g,
                                            float2 *lds_stat, f32x4 *lds_red) {
@@ -407,8 +405,13 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
     zero_row<D, KS, 4, SP>(lds_g);
     if (threadIdx.x == 0) lds_stat[G::ZROW] = make_float2(0.f, 0.f);
 
-    // wave = block of 4x4 keys (0..3) + 4 * (its part of the block's queries)
-    const int wave = (threadIdx.x >> 6) & 3, part = threadIdx.x >> 8;
+    // wave = block of 4x4 keys (0..3) + 4 * PART; part p takes reduction steps
+    // K0 = p * CH .. K1 - 1 (compile-time, so that every token's place in the halo and its
+    // mask fold to constants)
+    const int wave = SP == 1 ? threadIdx.x >> 6 : (threadIdx.x >> 6) & 3;
+    constexpr int part = PART;
+    constexpr int CH = (G::KSTEPS + SP - 1) / SP;
+    constexpr int K0 = PART * CH, K1 = K0 + CH < G::KSTEPS ? K0 + CH : G::KSTEPS;
     const int l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
     const int orow = (wave >> 1) * 4, ocol = (wave & 1) * 4;
@@ -514,11 +517,6 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
             dk[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
             dv[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-        // this wave's share of the reduction steps (all of them if SP == 1)
-        auto steps = [&](auto part_c) __attribute__((always_inline)) {
-        constexpr int CH = (G::KSTEPS + SP - 1) / SP;
-        constexpr int K0 = decltype(part_c)::value * CH;
-        constexpr int K1 = K0 + CH < G::KSTEPS ? K0 + CH : G::KSTEPS;
 #pragma unroll
         for (int ks = K0; ks < K1; ks++) {
             s16x8 pb, dsb;
@@ -560,23 +558,12 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
                                     dsb, dk[mt]);
             }
         }
-        };
-        if constexpr (SP == 1) {
-            steps(std::integral_constant<int, 0>{});
-        } else {
-            static_assert(SP == 2, "two parts");
-            if (part == 0) steps(std::integral_constant<int, 0>{});
-            else steps(std::integral_constant<int, 1>{});
-        }
 
-        auto store = [&]() __attribute__((always_inline)) {
-            const int kr = cur.r0 + orow + (n >> 2), kc = cur.c0 + ocol + (n & 3);
-            const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + kr) * s.W + kc;
+        const int kr = cur.r0 + orow + (n >> 2), kc = cur.c0 + ocol + (n & 3);
+        const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + kr) * s.W + kc;
+        if constexpr (SP == 1) {
             store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
             store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
-        };
-        if constexpr (SP == 1) {
-            store();
             if (!more) break;
             load_keys(nxt);
             __syncthreads();
@@ -584,6 +571,7 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
             // the second part hands its sums to the first through LDS; the first adds
             // and stores them once the barrier that ends the tile has passed (the
             // second part writes again only after the next tile's first barrier)
+            static_assert(SP <= 2, "two parts");
             f32x4 *red = lds_red + wave * 64 + l;
             if (part == 1) {
 #pragma unroll
@@ -600,7 +588,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
                     dk[mt] += red[mt * 256];
                     dv[mt] += red[(G::DT + mt) * 256];
                 }
-                store();
+                store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
+                store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
             }
             if (!more) break;
         }
@@ -829,10 +818,14 @@ __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (Geo<D, KS, 4, SP>::WAVES)
     __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
     // partial dK and dV of the second part of every block
     __shared__ f32x4 lds_red[SP > 1 ? 2 * G::DT * 256 : 1];
-    if ((int)blockIdx.x < inner_blocks)
-        dkdv_inner<BF, D, KS, ROLL, SP>(a, ts, n_inner, rp, blockIdx.x, inner_blocks, lds_q, lds_g,
-                                        lds_stat, lds_red);
-    else
+    if ((int)blockIdx.x < inner_blocks) {
+        if (SP == 1 || threadIdx.x < 256)
+            dkdv_inner<BF, D, KS, ROLL, SP, 0>(a, ts, n_inner, rp, blockIdx.x, inner_blocks, lds_q,
+                                               lds_g, lds_stat, lds_red);
+        else  // the same number of barriers as the first part
+            dkdv_inner<BF, D, KS, ROLL, SP, SP - 1>(a, ts, n_inner, rp, blockIdx.x, inner_blocks,
+                                                    lds_q, lds_g, lds_stat, lds_red);
+    } else
         dkdv_frame<BF, D, KS, SP>(a, ts, n_frame, blockIdx.x - inner_blocks,
                                   gridDim.x - inner_blocks, lds_q, lds_g, lds_stat, lds_red);
 }
@@ -977,7 +970,10 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             // of a frame tile in inner tiles: about 2 when the inner tiles are bound
             // by arithmetic (d <= 64), about 1.15 when they are bound by HBM (d = 128).
             constexpr int SP = kDkdvSplit<D, KS>, NT = Geo<D, KS, 4, SP>::NT;
-            const double cost = D >= 128 ? 1.15 : 2.0;
+#ifndef ENATTEN_FRAME_COST
+#define ENATTEN_FRAME_COST (D >= 128 ? 1.15 : 2.0)
+#endif
+            const double cost = ENATTEN_FRAME_COST;
             const int grid = persistent_grid<bwd_dkdv_mfma<BF, D, KS, false, SP>>(nb, NT);
             int inner_blocks = 0;
             if (n_frame == 0) {
