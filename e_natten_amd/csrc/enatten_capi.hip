@@ -302,6 +302,8 @@ int enatten1d_fwd(const void *q, const void *k, const void *v, void *o, float *l
     if ((rc = view_1d(fn, "o", o, o_strides, heads, T, D, &a.o))) return rc;
     a.lse = lse;
     a.s = Shape{B, heads, 1, T, D, 1, kernel_size, scale};  // a 1 x k window on a 1 x T image
+    if (g_path.load() != ENATTEN_PATH_SIMT && mfma1d_supported(D, kernel_size, dtype))
+        return launch_fwd1d_mfma(a, dtype, static_cast<hipStream_t>(stream));
     return launch_fwd_simt(a, dtype, static_cast<hipStream_t>(stream));
 }
 
@@ -333,6 +335,8 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, co
     a.delta = static_cast<float *>(workspace);
     a.zinv = a.delta + (size_t)B * heads * T;
     a.s = Shape{B, heads, 1, T, D, 1, kernel_size, scale};
+    if (g_path.load() != ENATTEN_PATH_SIMT && mfma1d_supported(D, kernel_size, dtype))
+        return launch_bwd1d_mfma(a, dtype, static_cast<hipStream_t>(stream));
     return launch_bwd_simt(a, dtype, static_cast<hipStream_t>(stream));
 }
 

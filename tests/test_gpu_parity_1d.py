@@ -61,6 +61,14 @@ def test_gradcheck_shape_of_reference():
     ((1, 1, 7, 8), 7, torch.float32),      # window == sequence
     ((1, 3, 19, 5), 3, torch.float32),     # odd head dim
     ((1, 2, 40, 16), 1, torch.bfloat16),
+    ((2, 2, 64, 128), 3, torch.bfloat16),    # exactly one tile
+    ((1, 3, 65, 64), 17, torch.bfloat16),    # a second tile of one position; largest 32-token window
+    ((1, 2, 200, 32), 19, torch.float16),    # 64-token windows
+    ((1, 1, 130, 64), 49, torch.bfloat16),   # largest window of the matrix-core kernels
+    ((1, 1, 49, 128), 49, torch.bfloat16),   # window == sequence
+    ((1, 2, 300, 128), 31, torch.bfloat16),
+    ((3, 2, 1000, 32), 5, torch.bfloat16),
+    ((1, 1, 120, 64), 51, torch.bfloat16),   # beyond them: general kernels
 ])
 def test_shapes_1d(shape, ks, dtype):
     _run(shape, dtype, ks, seed=2)
