@@ -64,6 +64,15 @@ __device__ __forceinline__ float col_sum(float x) {
     return x + __shfl_xor(x, 32, 64);
 }
 
+// 16 bytes of an output tensor, with a non-temporal store: outputs are written once and
+// never read by the kernel that writes them, and stores that do not allocate in L2 leave
+// it to the halo rows that neighbouring workgroups share (measured at B4 N4 128x128,
+// d=128, k=5: forward 60.9 -> 54.7 us, dQ pass 68.1 -> 61.5, dK/dV pass 96.2 -> 91.4, fused
+// backward 147.2 -> 142.7; the same for the read-once query rows was measured slower).
+__device__ __forceinline__ void store16(short *p, u32x4 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
+}
+
 // Stores one token's D output channels from the accumulators of the second product.
 // `acc[t][i]` is channel g*D/4 + t*4 + i of this lane's token (lanes l, l+16, l+32,
 // l+48 share a token, g = l/16): D/32 pieces of 16 bytes per lane.  Written as they
@@ -113,7 +122,7 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
         if (live) {
 #pragma unroll
             for (int j = 0; j < NP; j++)
-                *reinterpret_cast<u32x4 *>(token + j * (D / 4) + g * 8) = p[j];
+                store16(token + j * (D / 4) + g * 8, p[j]);
         }
     } else {
         // D = 32: the four lanes of a token already cover its 64 bytes.  D = 64 (pieces
@@ -121,7 +130,7 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
         if (live) {
 #pragma unroll
             for (int j = 0; j < NP; j++)
-                *reinterpret_cast<u32x4 *>(token + g * (D / 4) + j * 8) = p[j];
+                store16(token + g * (D / 4) + j * 8, p[j]);
         }
     }
 }

@@ -223,7 +223,7 @@ __device__ __forceinline__ void store32(float *token, int g, const f32x4 *acc, f
     if (!live) return;
 #pragma unroll
     for (int m = 0; m < D / 16; m++)
-        *reinterpret_cast<f32x4 *>(token + 16 * m + 4 * g) = acc[m] * mul;
+        __builtin_nontemporal_store(acc[m] * mul, reinterpret_cast<f32x4 *>(token + 16 * m + 4 * g));
 }
 
 __device__ __forceinline__ const float *image32(const View &v, const Tile &tl) {
