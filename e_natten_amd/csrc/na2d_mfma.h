@@ -175,10 +175,7 @@ struct Geo {
     //    instructions with it, LDS conflict cycles fall from 44-52% to 34-39% of the LDS
     //    cycles, and the kernels get 3-5% SLOWER (they wait on memory and instruction
     //    latency, not on LDS bandwidth, which is about a third used).  So it is off.
-#ifndef ENATTEN_SWZ_EXPR
-#define ENATTEN_SWZ_EXPR false
-#endif
-    static constexpr bool SWZ = ENATTEN_SWZ_EXPR;
+    static constexpr bool SWZ = false;
     static constexpr int PITCH = SWZ ? D : D + 8;  // LDS row pitch in elements
     static constexpr int ROWS = HR * HC + 1;      // + one all-zero row for padding tokens
     static constexpr int ZROW = HR * HC;

@@ -276,10 +276,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
             // the largest halos it is not kept but formed a second time once delta
             // is known (measured faster there: the matrix cores are idle, the
             // registers are not).
-#ifndef ENATTEN_KEEPDP_EXPR
-#define ENATTEN_KEEPDP_EXPR !(G::WAVES == 1 && G::MT >= 16)
-#endif
-            constexpr bool kKeepDp = ENATTEN_KEEPDP_EXPR;
+            constexpr bool kKeepDp = !(G::WAVES == 1 && G::MT >= 16);
             f32x4 dp[kKeepDp ? G::MT : 1];
             s16x8 dsb[G::KSTEPS];
             float dpart = 0.f;
@@ -861,20 +858,14 @@ constexpr bool kTallBuilt =
     D == 64 && KS >= 7 &&
     (size_t)2 * Geo<D, KS, 8>::ROWS * Geo<D, KS, 8>::PITCH * sizeof(short) <= 160 * 1024;
 template <int D, int KS>
-#ifndef ENATTEN_TALLDQ_MAXK
-#define ENATTEN_TALLDQ_MAXK 11
-#endif
-constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= ENATTEN_TALLDQ_MAXK;
+constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= 11;
 
 // The dK/dV pass with two waves per 4x4 block of keys, each on half of the block's
 // queries (Geo's SP): where the staged queries leave LDS for one workgroup per CU, a
 // SIMD then still holds two waves.  Built for head_dim 64 (the partial sums of the
 // second wave pass through 32 KB of LDS there).
-#ifndef ENATTEN_DKDV_SPLIT_EXPR
-#define ENATTEN_DKDV_SPLIT_EXPR (D == 64 && Geo<D, KS>::WAVES == 1 ? 2 : 1)
-#endif
 template <int D, int KS>
-constexpr int kDkdvSplit = ENATTEN_DKDV_SPLIT_EXPR;
+constexpr int kDkdvSplit = D == 64 && Geo<D, KS>::WAVES == 1 ? 2 : 1;
 
 template <bool BF, int D, int KS>
 int fwd_launch(const FwdArgs &a, hipStream_t st) {
@@ -970,10 +961,7 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             // of a frame tile in inner tiles: about 2 when the inner tiles are bound
             // by arithmetic (d <= 64), about 1.15 when they are bound by HBM (d = 128).
             constexpr int SP = kDkdvSplit<D, KS>, NT = Geo<D, KS, 4, SP>::NT;
-#ifndef ENATTEN_FRAME_COST
-#define ENATTEN_FRAME_COST (D >= 128 ? 1.15 : 2.0)
-#endif
-            const double cost = ENATTEN_FRAME_COST;
+            const double cost = D >= 128 ? 1.15 : 2.0;
             const int grid = persistent_grid<bwd_dkdv_mfma<BF, D, KS, false, SP>>(nb, NT);
             int inner_blocks = 0;
             if (n_frame == 0) {
