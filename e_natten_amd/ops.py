@@ -239,10 +239,60 @@ class Natten2d(torch.autograd.Function):
         return dQ, dK, dV, None, None
 
 
-def natten2d(q, k, v, kernel_size=7, scale=1.0):
+class Natten2dDilated(torch.autograd.Function):
+    """Dilated 2D neighborhood attention: query (x, y) attends the kernel_size^2 keys
+    that are `dilation` apart around it (NATTEN's dilated neighborhood; the reference
+    has no dilation and always passes 1 to its comparator, test.py:17).  Pixels with
+    equal (x mod dilation, y mod dilation) only ever see each other, and inside such
+    a sub-grid the rule is the plain one, so the operator is the undilated kernels run
+    on the dilation^2 strided sub-grids of q, k, v (the C ABI takes strides), each
+    writing its own pixels of the outputs."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V, kernel_size, scale, dilation):
+        o = torch.empty(Q.shape, dtype=Q.dtype, device=Q.device)
+        lses = []
+        for i in range(dilation):
+            for j in range(dilation):
+                sub = (slice(None), slice(None), slice(i, None, dilation), slice(j, None, dilation))
+                o_s, lse_s = torch.ops.enatten.na2d_fwd(Q[sub], K[sub], V[sub], kernel_size, scale)
+                o[sub] = o_s
+                lses.append(lse_s)
+        ctx.save_for_backward(Q, K, V, o, *lses)
+        ctx.args = (kernel_size, scale, dilation)
+        return o
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_output):
+        Q, K, V, o, *lses = ctx.saved_tensors
+        kernel_size, scale, dilation = ctx.args
+        dQ, dK, dV = (torch.empty(Q.shape, dtype=Q.dtype, device=Q.device) for _ in range(3))
+        for i in range(dilation):
+            for j in range(dilation):
+                sub = (slice(None), slice(None), slice(i, None, dilation), slice(j, None, dilation))
+                dq, dk, dv = torch.ops.enatten.na2d_bwd(Q[sub], K[sub], V[sub], o[sub],
+                                                        lses[i * dilation + j], grad_output[sub],
+                                                        kernel_size, scale)
+                dQ[sub], dK[sub], dV[sub] = dq, dk, dv
+        return dQ, dK, dV, None, None, None
+
+
+def natten2d(q, k, v, kernel_size=7, scale=1.0, dilation=1):
     """``natten2d(q, k, v, kernel_size) -> out`` on ``[B, heads, H, W, d]`` tensors,
     differentiable in q, k and v: the reference's entry point
-    (e_natten/triton.py:550, e_natten/__init__.py:1), positional like it."""
+    (e_natten/triton.py:550, e_natten/__init__.py:1), positional like it.
+    ``dilation`` > 1 spaces every neighborhood's keys that far apart (needs image sides
+    of at least kernel_size * dilation)."""
+    if dilation != 1:
+        if not isinstance(dilation, int) or isinstance(dilation, bool) or dilation < 1:
+            raise ValueError("dilation must be a positive int")
+        _validate(q, k, v, kernel_size)
+        _require_gpu(q, "natten2d")
+        if min(q.shape[2], q.shape[3]) < kernel_size * dilation:
+            raise ValueError("input of extent %dx%d is smaller than kernel_size * dilation = %d"
+                             % (q.shape[2], q.shape[3], kernel_size * dilation))
+        return Natten2dDilated.apply(q, k, v, kernel_size, float(scale), dilation)
     if not NATIVE_BINDING:
         return Natten2d.apply(q, k, v, kernel_size, scale)
     _validate(q, k, v, kernel_size)

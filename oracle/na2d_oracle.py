@@ -381,6 +381,62 @@ def natten2d_av(p, v, kernel_size: int) -> torch.Tensor:
 # --------------------------------------------------------------------------
 # error measures used by the parity tests
 # --------------------------------------------------------------------------
+# --------------------------------------------------------------------------
+# dilated neighborhoods (beyond the reference, which always passes dilation 1 to its
+# comparator: test.py:17,21)
+# --------------------------------------------------------------------------
+def dilated_win_start(i: int, L: int, k: int, dilation: int) -> int:
+    """First key of query i's window on an axis of length L: its k keys are
+    start, start + dilation, ..., start + (k - 1) * dilation.
+
+    Restates the window rule of the third-party NATTEN package (SHI-Labs; the
+    comparator the reference's test.py imports, absent here and un-pinned there) as
+    published in its CPU/CUDA sources, `get_window_start(index, length, kernel_size,
+    neighborhood_size, dilation)`: centred where it fits, otherwise the first /
+    last k positions of the query's residue class modulo the dilation.
+    """
+    ns = k // 2
+    if dilation <= 1:
+        return max(i - ns, 0) + (L - i - ns - 1 if i + ns >= L else 0)
+    ni = i - ns * dilation
+    if ni < 0:
+        return i % dilation
+    if i + ns * dilation >= L:
+        imodd = i % dilation
+        a = (L // dilation) * dilation
+        b = L - a
+        if imodd < b:
+            return L - b + imodd - 2 * ns * dilation
+        return a + imodd - k * dilation
+    return ni
+
+
+def dilated_neighbour_mask(H: int, W: int, k: int, dilation: int) -> torch.Tensor:
+    """[H*W, H*W] bool: query (row) attends key (column), from dilated_win_start."""
+    def axis(L):
+        m = torch.zeros(L, L, dtype=torch.bool)
+        for i in range(L):
+            s0 = dilated_win_start(i, L, k, dilation)
+            for j in range(k):
+                m[i, s0 + j * dilation] = True
+        return m
+    mr, mc = axis(H), axis(W)
+    return (mr[:, None, :, None] & mc[None, :, None, :]).reshape(H * W, H * W)
+
+
+def natten2d_dilated_dense_mask(q, k, v, kernel_size: int, dilation: int, scale: float = 1.0):
+    """O of dilated 2D neighborhood attention through torch's
+    scaled_dot_product_attention with the dense mask above; differentiable."""
+    B, N, H, W, D = q.shape
+    if H < kernel_size * dilation or W < kernel_size * dilation:
+        raise ValueError("image sides must be >= kernel_size * dilation")
+    m = dilated_neighbour_mask(H, W, kernel_size, dilation).to(q.device)
+    o = torch.nn.functional.scaled_dot_product_attention(
+        q.reshape(B, N, H * W, D), k.reshape(B, N, H * W, D), v.reshape(B, N, H * W, D),
+        attn_mask=m, scale=scale)
+    return o.reshape(B, N, H, W, D)
+
+
 def max_abs_err(x: torch.Tensor, ref: torch.Tensor) -> float:
     return (x.double() - ref.double()).abs().max().item()
 

@@ -464,3 +464,27 @@ def test_side_stream_and_graph_replay(_lib):
         for x, y in zip((o2, dq2, dk2, dv2), eager):
             assert torch.equal(x.cpu(), y)
         _ = (qs.float() @ qs.float().transpose(-1, -2)).sum().item()  # unrelated eager work
+
+
+@pytest.mark.parametrize("shape,ks,dil,dtype", [
+    ((1, 2, 20, 22, 32), 3, 2, BF),      # every sub-grid on the matrix-core kernels
+    ((2, 1, 31, 29, 64), 5, 3, BF),      # sub-grids of unequal sizes
+    ((1, 2, 24, 24, 128), 5, 4, F16),
+    ((1, 1, 14, 15, 8), 7, 2, F32),      # general kernels
+])
+def test_dilated_neighborhoods(shape, ks, dil, dtype, _lib):
+    # natten2d(..., dilation=d) against the dense-mask oracle built from NATTEN's dilated
+    # window rule (oracle/na2d_oracle.py: dilated_win_start), forward and backward
+    from e_natten_amd import natten2d
+    q, k, v, g = make_inputs(shape, dtype, seed=11)
+    print("case dilated", shape, dtype, "k=%d dilation=%d" % (ks, dil), flush=True)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    o_ref = O.natten2d_dilated_dense_mask(qr, kr, vr, ks, dil)
+    dq_ref, dk_ref, dv_ref = torch.autograd.grad(o_ref, (qr, kr, vr), g.double())
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = natten2d(qg, kg, vg, ks, 1.0, dil)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), g.cuda())
+    assert_close(tuple(t.detach().cpu() for t in (o, dq, dk, dv)),
+                 (o_ref.detach(), dq_ref, dk_ref, dv_ref), dtype, "dilated %s" % (shape,))
+    with pytest.raises(ValueError):
+        natten2d(qg, kg, vg, ks, 1.0, max(shape[2], shape[3]))

@@ -102,3 +102,24 @@ def test_unfused_comparator_equals_fused():
     for k in [3, 5, 7, 9, 11]:
         p = torch.softmax(O.natten2d_qk(q, kk, k), dim=-1)
         assert O.max_abs_err(O.natten2d_av(p, v, k), O.natten2d_gather(q, kk, v, k)) < 1e-12
+
+
+@pytest.mark.parametrize("H,W,ks,dil", [(12, 13, 3, 2), (15, 11, 3, 3), (21, 20, 5, 4), (9, 10, 3, 1)])
+def test_dilated_window_rule_is_the_plain_rule_on_residue_classes(H, W, ks, dil):
+    # NATTEN's dilated window start, restated in the oracle, against the statement the
+    # product relies on: pixels of one residue class modulo the dilation form a sub-grid
+    # on which the neighbourhood is the undilated one.
+    for L in (H, W):
+        for i in range(L):
+            r, t = i % dil, i // dil
+            Ls = (L - r + dil - 1) // dil
+            assert O.dilated_win_start(i, L, ks, dil) == r + dil * O.win_start(t, Ls, ks)
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(1, 2, H, W, 4, generator=g, dtype=torch.float64) for _ in range(3))
+    ref = O.natten2d_dilated_dense_mask(q, k, v, ks, dil)
+    got = torch.empty_like(ref)
+    for i in range(dil):
+        for j in range(dil):
+            sub = (slice(None), slice(None), slice(i, None, dil), slice(j, None, dil))
+            got[sub] = O.natten2d_gather(q[sub], k[sub], v[sub], ks)
+    assert torch.allclose(got, ref, atol=1e-12)
