@@ -806,8 +806,15 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 // every CU and end together.
 // SP = 2: eight waves, two per 4x4 block of keys (see Geo), for halos that leave LDS for
 // one workgroup per CU.
+// Waves per SIMD that the dK/dV pass budgets its registers for: three where LDS admits
+// three workgroups per CU (head_dim <= 64 with small halos; it fits 168 registers there,
+// measured 35 -> 32 us at B8 N2 112x112 d32 k7 and 67 -> 60 us at B4 N4 128x128 d32 k9;
+// the forward and the dQ pass spill under that budget and get slower).
+template <int D, int KS, int SP>
+constexpr int kDkdvWaves =
+    SP == 1 && D <= 64 && 3 * (Geo<D, KS>::LDS_BYTES + 2048) <= 160 * 1024 ? 3 : Geo<D, KS, 4, SP>::WAVES;
 template <bool BF, int D, int KS, bool ROLL, int SP = 1>
-__global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (Geo<D, KS, 4, SP>::WAVES)) void bwd_dkdv_mfma(
+__global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) void bwd_dkdv_mfma(
     BwdArgs a, TileSet ts, int n_inner, int n_frame, int inner_blocks, Runs rp) {
     using G = Geo<D, KS, 4, SP>;
     __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
