@@ -185,6 +185,9 @@ def main():
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run a plain 256 MiB device copy (calibrates rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--seq", type=int, default=0,
+                    help="time natten1d on [batch, heads, SEQ, head_dim] sequences instead of "
+                         "natten2d on images (no sweep, no unfused comparator, no CPU baseline)")
     ap.add_argument("--config", choices=sorted(CONFIGS),
                     help="one of the named benchmark configurations (sets the shape flags)")
     args = ap.parse_args()
@@ -196,8 +199,10 @@ def main():
                  "it has no cross-GPU path, batch*head slabs are independent")
 
     import torch
-    from e_natten_amd import _lib, kernel_path, natten2d
+    from e_natten_amd import _lib, kernel_path, natten1d, natten2d
     from e_natten_amd import build
+    if args.seq:
+        args.no_sweep = args.no_unfused = args.no_cpu = True
     if not (os.path.exists(_lib.LIB_PATH) and os.path.exists(build.TORCH_LIB)):
         build.build()
     lib = _lib.load()
@@ -209,7 +214,8 @@ def main():
         lib.enatten_set_path(_lib.PATH_MFMA_SPLIT)
     dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype]
     B, N, S, D, ks = args.batch, args.heads, args.side, args.head_dim, args.kernel_size
-    shape = (B, N, S, S, D)
+    shape = (B, N, args.seq, D) if args.seq else (B, N, S, S, D)
+    op = natten1d if args.seq else natten2d
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(0)
     sets, cold = rotating_sets(shape, dtype, dev, 4)
@@ -220,7 +226,7 @@ def main():
 
     def step(i=0):
         q, k, v, d_o = sets[i % len(sets)]
-        o = natten2d(q, k, v, ks)
+        o = op(q, k, v, ks)
         return torch.autograd.grad(o, (q, k, v), d_o)
 
     for i in range(args.warmup):
@@ -256,9 +262,11 @@ def main():
         torch.cuda.synchronize()
 
     ms_step = elapsed * 1e3 / args.steps
-    queries = B * N * S * S
-    useful = 14.0 * ks * ks * D * queries
-    alg = algorithmic_bytes(B, N, S, S, D, q.element_size())
+    queries = B * N * (args.seq if args.seq else S * S)
+    window = ks if args.seq else ks * ks
+    useful = 14.0 * window * D * queries
+    alg = (algorithmic_bytes(B, N, 1, args.seq, D, q.element_size()) if args.seq
+           else algorithmic_bytes(B, N, S, S, D, q.element_size()))
 
     kern = {}
     for i, name in enumerate(KERNELS):
@@ -276,7 +284,9 @@ def main():
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
     if os.path.exists(tpath):
-        rec = json.load(open(tpath)).get("%s/side%d/%s" % (kern[dom]["kernel"], S, args.dtype))
+        # counter figures of this very workload, where a profile of it has been taken
+        rec = json.load(open(tpath)).get("%s/B%d_N%d_Q%d_d%d_k%d_e%d" % (
+            kern[dom]["kernel"], B, N, queries // (B * N), D, window, q.element_size()))
         traffic = rec["bytes_per_launch"] if rec else None
     kernel_ms = sum(kern[n]["avg_us"] for n in names) / 1e3
     roofline = {
@@ -288,12 +298,16 @@ def main():
         "path_frac": alg["path"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
     }
     path = kernel_path(D, ks, dtype)
+    if args.seq:   # the 1D matrix-core kernels: bf16 / f16, head_dim 32 / 64 / 128, kernel_size <= 49
+        path = "mfma" if path != "none" and args.dtype != "fp32" and D in (32, 64, 128) and 3 <= ks <= 49 \
+            else "simt"
     if path == "mfma" and args.dtype in MFMA_PEAK_TF and not args.simt:
         # useful FLOPs against the matrix-core peak of the dtype the kernels compute in
         roofline["mfma_frac_useful"] = useful / (kernel_ms * 1e-3) / 1e12 / MFMA_PEAK_TF[args.dtype]
-    working_set = 8 * B * N * S * S * D * q.element_size()   # q, k, v, o, dO, dq, dk, dv
+    working_set = 8 * queries * D * q.element_size()   # q, k, v, o, dO, dq, dk, dv
     out = {
-        "metric": "natten2d fwd+bwd useful TFLOP/s (B%d H%d d%d k%d %s)" % (B, N, D, ks, args.dtype),
+        "metric": "%s fwd+bwd useful TFLOP/s (B%d H%d d%d k%d %s)"
+                  % ("natten1d" if args.seq else "natten2d", B, N, D, ks, args.dtype),
         "value": useful / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
         "timing": "cold: %d input sets in rotation (%s twice the 256 MB memory-side cache)"
@@ -304,8 +318,10 @@ def main():
         "kernel_event_sampling": "every %d-th launch" % period,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": "natten2d fwd+bwd B=%d heads=%d H=W=%d head_dim=%d kernel_size=%d"
-                               % (B, N, S, D, ks),
+        "config": {"workload": ("natten1d fwd+bwd B=%d heads=%d T=%d head_dim=%d kernel_size=%d"
+                                % (B, N, args.seq, D, ks)) if args.seq else
+                               ("natten2d fwd+bwd B=%d heads=%d H=W=%d head_dim=%d kernel_size=%d"
+                                % (B, N, S, D, ks)),
                    "kernel_path": "simt" if args.simt else path, "queries": queries,
                    "useful_gflop": useful / 1e9},
         "roofline": roofline,
