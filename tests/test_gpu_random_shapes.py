@@ -1,0 +1,87 @@
+"""Seeded random shapes through the C ABI against the CPU oracle: every kernel family
+(16-bit matrix-core, float32 matrix-core, 1D matrix-core, general), both backward paths,
+ragged and tile-aligned images, batch * heads from 1 to hundreds."""
+import random
+
+import pytest
+import torch
+
+from _util import BF16_REL, FP32_MAX_ABS, O, ensure_built, make_inputs, oracle_all, run_capi
+from oracle import na1d_oracle as O1
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib():
+    assert torch.cuda.is_available()
+    return ensure_built()
+
+
+def _cases_2d(n, seed):
+    rnd = random.Random(seed)
+    out = []
+    for it in range(n):
+        dt = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+        D = rnd.choice([32, 64, 64, 128, 128, 48] if dt != torch.float32 else [32, 64, 128, 128, 24])
+        ks = rnd.choice([3, 5, 5, 7, 7, 9, 11, 13] if dt != torch.float32 else [3, 5, 5, 7, 9])
+        H, W = rnd.randint(ks, 70), rnd.randint(ks, 70)
+        if rnd.random() < 0.4:
+            H, W = max(ks, (H + 7) // 8 * 8), max(ks, (W + 7) // 8 * 8)
+        bn = max(1, int(rnd.choice([3e4, 1.5e5, 4e5]) / (H * W)))
+        B = rnd.choice([1, 2, 4])
+        N = max(1, bn // B)
+        out.append(((B, N, H, W, D), ks, dt, rnd.choice([0, 0, 3, 4]), it))
+    return out
+
+
+@pytest.mark.parametrize("shape,ks,dtype,path,seed", _cases_2d(28, 2024))
+def test_random_shapes_2d(shape, ks, dtype, path, seed, lib):
+    prev = lib.enatten_set_path(path)
+    try:
+        print("case random", shape, "k=%d" % ks, dtype, "path", path, flush=True)
+        q, k, v, g = make_inputs(shape, dtype, seed=100 + seed)
+        o, lse, dq, dk, dv = run_capi(q, k, v, g, ks)
+        ref = oracle_all(q, k, v, g, ks)
+        for name, x, r in zip(("O", "dQ", "dK", "dV"), (o, dq, dk, dv), (ref[0], ref[2], ref[3], ref[4])):
+            assert torch.isfinite(x.float()).all(), name
+            if dtype == torch.float32:
+                assert O.max_abs_err(x, r) <= FP32_MAX_ABS, (name, O.max_abs_err(x, r))
+            else:
+                assert O.rel_err(x, r) <= BF16_REL, (name, O.rel_err(x, r))
+        assert (lse - ref[1]).abs().max().item() <= (1e-4 if dtype == torch.float32 else 2e-2)
+    finally:
+        lib.enatten_set_path(prev)
+
+
+def _cases_1d(n, seed):
+    rnd = random.Random(seed)
+    out = []
+    for it in range(n):
+        dt = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+        D = rnd.choice([32, 64, 128, 16])
+        ks = rnd.choice([3, 5, 7, 9, 13, 17, 19, 25, 33, 49, 51])
+        T = rnd.randint(ks, 700)
+        B, N = rnd.choice([1, 2, 3]), rnd.choice([1, 2, 5])
+        out.append(((B, N, T, D), ks, dt, it))
+    return out
+
+
+@pytest.mark.parametrize("shape,ks,dtype,seed", _cases_1d(16, 7))
+def test_random_shapes_1d(shape, ks, dtype, seed, lib):
+    from e_natten_amd import Natten1d
+    print("case random 1d", shape, "k=%d" % ks, dtype, flush=True)
+    g = torch.Generator().manual_seed(200 + seed)
+    q, k, v, d_o = (torch.randn(shape, generator=g).to(dtype) for _ in range(4))
+    ref = O1.natten1d_explicit(q, k, v, d_o, ks)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = Natten1d.apply(qg, kg, vg, ks, 1.0)
+    o.backward(d_o.cuda())
+    for name, x, r in zip(("O", "dQ", "dK", "dV"), (o, qg.grad, kg.grad, vg.grad),
+                          (ref[0], ref[2], ref[3], ref[4])):
+        x = x.detach().cpu()
+        assert torch.isfinite(x.float()).all(), name
+        if dtype == torch.float32:
+            assert O.max_abs_err(x, r) <= FP32_MAX_ABS, (name, O.max_abs_err(x, r))
+        else:
+            assert O.rel_err(x, r) <= BF16_REL, (name, O.rel_err(x, r))
