@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define ENATTEN_ABI_VERSION 2
+#define ENATTEN_ABI_VERSION 3
 
 /* element types of q, k, v, o and the gradients */
 enum { ENATTEN_F32 = 0, ENATTEN_BF16 = 1, ENATTEN_F16 = 2 };

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol(lib):
     for n in names:
         assert hasattr(lib, n), "libenatten.so does not export %s" % n
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.enatten_abi_version() == _lib.ABI_VERSION == 2
+    assert lib.enatten_abi_version() == _lib.ABI_VERSION == 3
 
 
 def test_c_abi_validates_before_launch(lib):
