@@ -69,6 +69,7 @@ def test_gradcheck_shape_of_reference():
     ((1, 2, 300, 128), 31, torch.bfloat16),
     ((3, 2, 1000, 32), 5, torch.bfloat16),
     ((1, 1, 120, 64), 51, torch.bfloat16),   # beyond them: general kernels
+    ((1, 2, 1 << 18, 32), 7, torch.bfloat16),  # a long sequence: 4096 tiles per (batch, head)
 ])
 def test_shapes_1d(shape, ks, dtype):
     _run(shape, dtype, ks, seed=2)

@@ -31,18 +31,18 @@ def _cases_2d(n, seed):
         bn = max(1, int(rnd.choice([3e4, 1.5e5, 4e5]) / (H * W)))
         B = rnd.choice([1, 2, 4])
         N = max(1, bn // B)
-        out.append(((B, N, H, W, D), ks, dt, rnd.choice([0, 0, 3, 4]), it))
+        out.append(((B, N, H, W, D), ks, dt, rnd.choice([0, 0, 3, 4]), rnd.choice([1.0, 1.0, 0.5, D ** -0.5]), it))
     return out
 
 
-@pytest.mark.parametrize("shape,ks,dtype,path,seed", _cases_2d(28, 2024))
-def test_random_shapes_2d(shape, ks, dtype, path, seed, lib):
+@pytest.mark.parametrize("shape,ks,dtype,path,scale,seed", _cases_2d(28, 2024))
+def test_random_shapes_2d(shape, ks, dtype, path, scale, seed, lib):
     prev = lib.enatten_set_path(path)
     try:
-        print("case random", shape, "k=%d" % ks, dtype, "path", path, flush=True)
+        print("case random", shape, "k=%d" % ks, dtype, "path", path, "scale", scale, flush=True)
         q, k, v, g = make_inputs(shape, dtype, seed=100 + seed)
-        o, lse, dq, dk, dv = run_capi(q, k, v, g, ks)
-        ref = oracle_all(q, k, v, g, ks)
+        o, lse, dq, dk, dv = run_capi(q, k, v, g, ks, scale)
+        ref = oracle_all(q, k, v, g, ks, scale)
         for name, x, r in zip(("O", "dQ", "dK", "dV"), (o, dq, dk, dv), (ref[0], ref[2], ref[3], ref[4])):
             assert torch.isfinite(x.float()).all(), name
             if dtype == torch.float32:
