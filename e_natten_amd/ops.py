@@ -320,9 +320,49 @@ class Natten1d(torch.autograd.Function):
         return dQ, dK, dV, None, None
 
 
-def natten1d(q, k, v, kernel_size=7, scale=1.0):
+class Natten1dDilated(torch.autograd.Function):
+    """Dilated 1D neighborhood attention: the undilated kernels on the `dilation`
+    strided sub-sequences (see Natten2dDilated)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, kernel_size, scale, dilation):
+        o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        lses = []
+        for i in range(dilation):
+            sub = (slice(None), slice(None), slice(i, None, dilation))
+            o_s, lse_s = torch.ops.enatten.na1d_fwd(q[sub], k[sub], v[sub], kernel_size, scale)
+            o[sub] = o_s
+            lses.append(lse_s)
+        ctx.save_for_backward(q, k, v, o, *lses)
+        ctx.args = (kernel_size, scale, dilation)
+        return o
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_output):
+        q, k, v, o, *lses = ctx.saved_tensors
+        kernel_size, scale, dilation = ctx.args
+        dQ, dK, dV = (torch.empty(q.shape, dtype=q.dtype, device=q.device) for _ in range(3))
+        for i in range(dilation):
+            sub = (slice(None), slice(None), slice(i, None, dilation))
+            dq, dk, dv = torch.ops.enatten.na1d_bwd(q[sub], k[sub], v[sub], o[sub], lses[i],
+                                                    grad_output[sub], kernel_size, scale)
+            dQ[sub], dK[sub], dV[sub] = dq, dk, dv
+        return dQ, dK, dV, None, None, None
+
+
+def natten1d(q, k, v, kernel_size=7, scale=1.0, dilation=1):
     """``natten1d(q, k, v, kernel_size) -> out`` on ``[B, heads, T, d]`` tensors
-    (e_natten/triton.py:485, e_natten/__init__.py:1)."""
+    (e_natten/triton.py:485, e_natten/__init__.py:1).  ``dilation`` as in natten2d."""
+    if dilation != 1:
+        if not isinstance(dilation, int) or isinstance(dilation, bool) or dilation < 1:
+            raise ValueError("dilation must be a positive int")
+        _validate(q, k, v, kernel_size, 4)
+        _require_gpu(q, "natten1d")
+        if q.shape[2] < kernel_size * dilation:
+            raise ValueError("sequence of %d positions is shorter than kernel_size * dilation = %d"
+                             % (q.shape[2], kernel_size * dilation))
+        return Natten1dDilated.apply(q, k, v, kernel_size, float(scale), dilation)
     if not NATIVE_BINDING:
         return Natten1d.apply(q, k, v, kernel_size, scale)
     _validate(q, k, v, kernel_size, 4)

@@ -95,3 +95,27 @@ def test_strided_and_contract_1d():
     assert O.rel_err(o.cpu(), ref) < BF16_REL
     with pytest.raises(ValueError):
         natten1d(dev[:, :, 0], dev[:, :, 1], dev[:, :, 2], 4)
+
+
+@pytest.mark.parametrize("shape,ks,dil,dtype", [((2, 2, 150, 64), 7, 3, torch.bfloat16),
+                                                ((1, 3, 61, 16), 5, 2, torch.float32)])
+def test_dilated_1d(shape, ks, dil, dtype):
+    # against a dense banded mask built from NATTEN's dilated window rule
+    from e_natten_amd import natten1d
+    g = torch.Generator().manual_seed(6)
+    q, k, v, d_o = (torch.randn(shape, generator=g).to(dtype) for _ in range(4))
+    T = shape[2]
+    m = torch.zeros(T, T, dtype=torch.bool)
+    for i in range(T):
+        s0 = O.dilated_win_start(i, T, ks, dil)
+        m[i, s0:s0 + ks * dil:dil] = True
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    o_ref = torch.nn.functional.scaled_dot_product_attention(qr, kr, vr, attn_mask=m, scale=1.0)
+    refs = (o_ref,) + torch.autograd.grad(o_ref, (qr, kr, vr), d_o.double())
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = natten1d(qg, kg, vg, ks, 1.0, dil)
+    got = (o,) + torch.autograd.grad(o, (qg, kg, vg), d_o.cuda())
+    for name, x, r in zip(("O", "dQ", "dK", "dV"), got, refs):
+        x, r = x.detach().cpu(), r.detach()
+        err = O.max_abs_err(x, r) if dtype == torch.float32 else O.rel_err(x, r)
+        assert err <= (FP32_MAX_ABS if dtype == torch.float32 else BF16_REL), (name, err)
