@@ -30,18 +30,11 @@ struct Geo1 {
     static constexpr int KSMAX = NKP - 15;         // largest kernel_size served
     static constexpr int HR = TW + KSMAX - 1;      // staged key rows (forward, dQ)
     static constexpr int RQ = TW + KSMAX - 1 + KSMAX / 2;  // staged query rows (dK/dV)
-    static constexpr int PITCH = D + 8;
-    static constexpr int CPR = D / 8;              // 16-byte chunks per row
-    static constexpr int RPP = 256 / CPR;          // rows staged per pass of the workgroup
-    static constexpr int NL = (HR * CPR + 255) / 256;
-    static constexpr int NLQ = (RQ * CPR + 255) / 256;
-    static constexpr int MT = NKP / 16;
-    static constexpr int KSTEPS = NKP / 32;
-    static constexpr int DS = D / 32;
-    static constexpr int DT = D / 16;
-    static constexpr size_t LDS_FWD = (size_t)2 * (HR + 1) * PITCH * sizeof(short);
-    static constexpr size_t LDS_DKDV = (size_t)2 * (RQ + 1) * PITCH * sizeof(short) + (RQ + 1) * 8;
-    static constexpr int WAVES = 2;                // waves per SIMD to budget registers for
+    static constexpr int PITCH = D + 8;            // LDS row pitch in elements (16-byte pad)
+    static constexpr int MT = NKP / 16;            // 16-token MFMA row tiles
+    static constexpr int KSTEPS = NKP / 32;        // reduction steps of the second product
+    static constexpr int DS = D / 32;              // reduction steps over channels
+    static constexpr int DT = D / 16;              // 16-channel row tiles of the output
 };
 
 // A tile of 64 positions of one (batch, head) sequence.
