@@ -58,7 +58,10 @@ void validate(const char *what, const Tensor &q, const Tensor &k, const Tensor &
     TORCH_CHECK_VALUE(q.numel() > 0, what, ": empty tensors are not supported");
     TORCH_CHECK_VALUE(q.size(-1) <= 1024, what, ": head_dim ", q.size(-1),
                       " exceeds the supported maximum of 1024");
-    TORCH_CHECK(q.is_cuda(), what, ": tensors must be on the GPU; this build has no CPU path");
+    // meta tensors (shape inference under tracing) pass: every operator returns outputs of
+    // the right shape for them without touching the library
+    TORCH_CHECK(q.is_cuda() || q.is_meta(), what,
+                ": tensors must be on the GPU; this build has no CPU path");
 }
 
 // The kernels take any strides on the leading axes but need unit stride on the
@@ -84,6 +87,9 @@ void check_bwd_extras(const char *what, const Tensor &q, const Tensor &o, const 
 std::tuple<Tensor, Tensor> na2d_fwd(const Tensor &q_, const Tensor &k_, const Tensor &v_,
                                     int64_t ks, double scale) {
     validate("enatten::na2d_fwd", q_, k_, v_, ks, 5);
+    if (q_.is_meta())
+        return {at::empty_like(kernel_layout(q_)),
+                at::empty({q_.size(0), q_.size(1), q_.size(2), q_.size(3)}, q_.options().dtype(at::kFloat))};
     const c10::DeviceGuard guard(q_.device());
     const Tensor q = kernel_layout(q_), k = kernel_layout(k_), v = kernel_layout(v_);
     const int B = q.size(0), N = q.size(1), H = q.size(2), W = q.size(3), D = q.size(4);
@@ -104,6 +110,10 @@ std::tuple<Tensor, Tensor, Tensor> na2d_bwd(const Tensor &q_, const Tensor &k_, 
                                             const Tensor &d_o_, int64_t ks, double scale) {
     validate("enatten::na2d_bwd", q_, k_, v_, ks, 5);
     check_bwd_extras("enatten::na2d_bwd", q_, o_, d_o_);
+    if (q_.is_meta()) {
+        const Tensor g = at::empty(q_.sizes(), q_.options());
+        return {g, at::empty_like(g), at::empty_like(g)};
+    }
     const c10::DeviceGuard guard(q_.device());
     const Tensor q = kernel_layout(q_), k = kernel_layout(k_), v = kernel_layout(v_);
     const Tensor o = kernel_layout(o_), d_o = kernel_layout(d_o_), lse = lse_.contiguous();
@@ -124,6 +134,9 @@ std::tuple<Tensor, Tensor, Tensor> na2d_bwd(const Tensor &q_, const Tensor &k_, 
 std::tuple<Tensor, Tensor> na1d_fwd(const Tensor &q_, const Tensor &k_, const Tensor &v_,
                                     int64_t ks, double scale) {
     validate("enatten::na1d_fwd", q_, k_, v_, ks, 4);
+    if (q_.is_meta())
+        return {at::empty_like(kernel_layout(q_)),
+                at::empty({q_.size(0), q_.size(1), q_.size(2)}, q_.options().dtype(at::kFloat))};
     const c10::DeviceGuard guard(q_.device());
     const Tensor q = kernel_layout(q_), k = kernel_layout(k_), v = kernel_layout(v_);
     const int B = q.size(0), N = q.size(1), T = q.size(2), D = q.size(3);
@@ -142,6 +155,10 @@ std::tuple<Tensor, Tensor, Tensor> na1d_bwd(const Tensor &q_, const Tensor &k_, 
                                             const Tensor &d_o_, int64_t ks, double scale) {
     validate("enatten::na1d_bwd", q_, k_, v_, ks, 4);
     check_bwd_extras("enatten::na1d_bwd", q_, o_, d_o_);
+    if (q_.is_meta()) {
+        const Tensor g = at::empty(q_.sizes(), q_.options());
+        return {g, at::empty_like(g), at::empty_like(g)};
+    }
     const c10::DeviceGuard guard(q_.device());
     const Tensor q = kernel_layout(q_), k = kernel_layout(k_), v = kernel_layout(v_);
     const Tensor o = kernel_layout(o_), d_o = kernel_layout(d_o_), lse = lse_.contiguous();
@@ -159,6 +176,32 @@ std::tuple<Tensor, Tensor, Tensor> na1d_bwd(const Tensor &q_, const Tensor &k_, 
     return {dq, dk, dv};
 }
 
+// The composite operators reach the four kernels' operators through the dispatcher, not
+// by a C++ call: tensor subclasses and modes above the backend keys (fake tensors under
+// torch.compile, functorch wrappers) then see them as opaque operators with a meta kernel.
+std::tuple<Tensor, Tensor> call_fwd(bool two_d, const Tensor &q, const Tensor &k, const Tensor &v,
+                                    int64_t ks, double scale) {
+    using Sig = std::tuple<Tensor, Tensor>(const Tensor &, const Tensor &, const Tensor &, int64_t,
+                                           double);
+    static const auto op2 =
+        c10::Dispatcher::singleton().findSchemaOrThrow("enatten::na2d_fwd", "").typed<Sig>();
+    static const auto op1 =
+        c10::Dispatcher::singleton().findSchemaOrThrow("enatten::na1d_fwd", "").typed<Sig>();
+    return (two_d ? op2 : op1).call(q, k, v, ks, scale);
+}
+std::tuple<Tensor, Tensor, Tensor> call_bwd(bool two_d, const Tensor &q, const Tensor &k,
+                                            const Tensor &v, const Tensor &o, const Tensor &lse,
+                                            const Tensor &d_o, int64_t ks, double scale) {
+    using Sig = std::tuple<Tensor, Tensor, Tensor>(const Tensor &, const Tensor &, const Tensor &,
+                                                   const Tensor &, const Tensor &, const Tensor &,
+                                                   int64_t, double);
+    static const auto op2 =
+        c10::Dispatcher::singleton().findSchemaOrThrow("enatten::na2d_bwd", "").typed<Sig>();
+    static const auto op1 =
+        c10::Dispatcher::singleton().findSchemaOrThrow("enatten::na1d_bwd", "").typed<Sig>();
+    return (two_d ? op2 : op1).call(q, k, v, o, lse, d_o, ks, scale);
+}
+
 // One autograd node for both operators: the forward keeps (q, k, v, o, lse), the
 // backward returns (dQ, dK, dV) and no gradient for kernel_size and scale.
 template <bool TWO_D>
@@ -167,7 +210,7 @@ struct NattenFn : public torch::autograd::Function<NattenFn<TWO_D>> {
                           int64_t ks, double scale) {
         at::AutoDispatchBelowADInplaceOrView below;
         Tensor o, lse;
-        std::tie(o, lse) = TWO_D ? na2d_fwd(q, k, v, ks, scale) : na1d_fwd(q, k, v, ks, scale);
+        std::tie(o, lse) = call_fwd(TWO_D, q, k, v, ks, scale);
         ctx->save_for_backward({q, k, v, o, lse});
         ctx->saved_data["kernel_size"] = ks;
         ctx->saved_data["scale"] = scale;
@@ -179,8 +222,7 @@ struct NattenFn : public torch::autograd::Function<NattenFn<TWO_D>> {
         const double scale = ctx->saved_data["scale"].toDouble();
         at::AutoDispatchBelowADInplaceOrView below;
         Tensor dq, dk, dv;
-        std::tie(dq, dk, dv) = TWO_D ? na2d_bwd(s[0], s[1], s[2], s[3], s[4], grads[0], ks, scale)
-                                     : na1d_bwd(s[0], s[1], s[2], s[3], s[4], grads[0], ks, scale);
+        std::tie(dq, dk, dv) = call_bwd(TWO_D, s[0], s[1], s[2], s[3], s[4], grads[0], ks, scale);
         return {dq, dk, dv, Tensor(), Tensor()};
     }
 };
@@ -194,10 +236,10 @@ Tensor natten1d_autograd(const Tensor &q, const Tensor &k, const Tensor &v, int6
     return NattenFn<false>::apply(q, k, v, ks, scale);
 }
 Tensor natten2d_plain(const Tensor &q, const Tensor &k, const Tensor &v, int64_t ks, double scale) {
-    return std::get<0>(na2d_fwd(q, k, v, ks, scale));
+    return std::get<0>(call_fwd(true, q, k, v, ks, scale));
 }
 Tensor natten1d_plain(const Tensor &q, const Tensor &k, const Tensor &v, int64_t ks, double scale) {
-    return std::get<0>(na1d_fwd(q, k, v, ks, scale));
+    return std::get<0>(call_fwd(false, q, k, v, ks, scale));
 }
 
 }  // namespace

@@ -488,3 +488,29 @@ def test_dilated_neighborhoods(shape, ks, dil, dtype, _lib):
                  (o_ref.detach(), dq_ref, dk_ref, dv_ref), dtype, "dilated %s" % (shape,))
     with pytest.raises(ValueError):
         natten2d(qg, kg, vg, ks, 1.0, max(shape[2], shape[3]))
+
+
+def test_traced_by_torch_compile(_lib):
+    # The operators are opaque to the tracer and carry meta kernels, so a function that
+    # calls them compiles as one graph (no graph break); the compiled function runs the same
+    # kernels, so forward and gradients equal the eager ones bit for bit.
+    from e_natten_amd import natten1d, natten2d, ops
+    if not ops.NATIVE_BINDING:
+        pytest.skip("native torch binding not built")
+
+    def f(q, k, v, s):
+        a = natten2d(q * 1.0, k, v, 5)
+        b = natten1d(s, s, s, 7)
+        return (a.float() ** 2).sum() + b.float().sum()
+
+    q, k, v, _ = make_inputs((2, 2, 24, 24, 64), BF, seed=5)
+    q, k, v = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    s = torch.randn(2, 2, 200, 32, device="cuda", dtype=F16, requires_grad=True)
+    ref = f(q, k, v, s)
+    gref = torch.autograd.grad(ref, (q, k, v, s))
+    fc = torch.compile(f, backend="aot_eager", fullgraph=True)
+    out = fc(q, k, v, s)
+    got = torch.autograd.grad(out, (q, k, v, s))
+    assert torch.equal(out.detach(), ref.detach())
+    for a, b in zip(got, gref):
+        assert torch.equal(a, b)

@@ -180,3 +180,22 @@ def test_product_package_does_not_import_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower() or f == "never", (f, "mentions the oracle")
+
+
+def test_meta_tensors_give_shapes_without_a_gpu():
+    # shape inference for tracing: the native operators accept meta tensors, validate them
+    # like real ones and return outputs (and gradients) of the right shape and dtype
+    from e_natten_amd import natten1d, natten2d, ops
+    if not ops.NATIVE_BINDING:
+        pytest.skip("native torch binding not built")
+    q = torch.empty(2, 3, 16, 12, 64, device="meta", dtype=torch.bfloat16, requires_grad=True)
+    o = natten2d(q, q, q, 5)
+    assert o.shape == q.shape and o.dtype == q.dtype and o.device.type == "meta"
+    (g,) = torch.autograd.grad(o, q, torch.empty_like(o))
+    assert g.shape == q.shape
+    o2, lse = torch.ops.enatten.na2d_fwd(q.detach(), q.detach(), q.detach(), 5, 1.0)
+    assert lse.shape == q.shape[:-1] and lse.dtype == torch.float32
+    s = torch.empty(2, 3, 100, 32, device="meta", dtype=torch.float16)
+    assert natten1d(s, s, s, 7).shape == s.shape
+    with pytest.raises(ValueError):
+        natten2d(q, q, q, 4)
