@@ -47,10 +47,8 @@ struct FGeo {
     }
     static constexpr int NL = q_passes(BR);               // chunks per thread and tensor (query side)
     // Key side beside the border: the queries that attend to a wave's 4x4 keys
-    // span up to SW + k/2 rows and columns there; they are numbered 16 per row.
+    // span up to SW + k/2 rows and columns there.
     static constexpr int SWB = G::SW + KS / 2;
-    static constexpr int MTB = (SWB + 1) / 2 * 2;         // one MFMA row tile per row, even
-    static constexpr int KSB = MTB / 2;
     static constexpr size_t LDS_BYTES =
         (size_t)4 * G::ROWS * G::PITCH * sizeof(short) + (size_t)G::ROWS * sizeof(float2);
     static constexpr bool FITS = LDS_BYTES <= 160 * 1024 && G::HR - BR <= BR && SWB <= 16 &&
@@ -192,12 +190,11 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     // they would hold registers through the math of a whole tile.
     // `side` (a compile-time 0 or 1) is the side of the calling wave: the key-side waves
     // then provably never touch the chunk registers beyond their share.
-    auto fetch = [&](Chunks<F::NL> &reg, const View &vw, const Tile &tl, int y0, int bc, auto nr,
+    auto fetch = [&](Chunks<F::NL> &reg, const View &vw, const char *base, int y0, int bc, auto nr,
                      auto side) __attribute__((always_inline)) {
         constexpr int NR = decltype(nr)::value;
         constexpr int SIDE = decltype(side)::value;
         constexpr int MINE = SIDE == 0 ? F::q_passes(NR) : F::passes(NR) - F::q_passes(NR);
-        const char *base = reinterpret_cast<const char *>(image<short>(vw, tl));
         const unsigned sh2 = (unsigned)vw.sh * 2u, sw2 = (unsigned)vw.sw * 2u;
 #pragma unroll
         for (int i = 0; i < MINE; i++) {
@@ -214,28 +211,41 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     // The loads of a step are issued in five parts (one tensor each) spread over the
     // math of the current tile: a CU only takes so many vector loads at a time, and a
     // wave that waits at the queue with all of them at once does no math meanwhile.
-    auto fetch_part = [&](const Tile &tl, int part, int y0, int bc, auto nr, auto side)
-                          __attribute__((always_inline)) {
+    // The image that is being staged: the start of its (batch, head) slice in every tensor.
+    // Kept per image, not formed per tile: the tensors' pointers and outer strides are then
+    // only needed where a run crosses into another image.
+    const char *img_q, *img_k, *img_v, *img_g, *img_o;
+    const float *img_lse;
+    auto set_image = [&](const Tile &tl) __attribute__((always_inline)) {
+        img_q = reinterpret_cast<const char *>(image<short>(a.q, tl));
+        img_k = reinterpret_cast<const char *>(image<short>(a.k, tl));
+        img_v = reinterpret_cast<const char *>(image<short>(a.v, tl));
+        img_g = reinterpret_cast<const char *>(image<short>(a.d_o, tl));
+        img_o = reinterpret_cast<const char *>(image<short>(a.o, tl));
+        img_lse = a.lse + ((int64_t)tl.bb * s.N + tl.nn) * s.H * (int64_t)s.W;
+    };
+    auto fetch_part = [&](int part, int y0, int bc, auto nr, auto side) __attribute__((always_inline)) {
         constexpr int NR = decltype(nr)::value;
-        const int64_t img_tok = ((int64_t)tl.bb * s.N + tl.nn) * s.H * (int64_t)s.W;
         if (part == 0) {
-            fetch(qst, a.q, tl, y0, bc, nr, side);
+            fetch(qst, a.q, img_q, y0, bc, nr, side);
             const int id = min(stid, NR * G::HC - 1);
             const int y = min(max(y0 + id / G::HC, 0), s.H - 1), x = min(max(bc + id % G::HC, 0), s.W - 1);
-            lse_st = a.lse[img_tok + (int64_t)y * s.W + x];
+            lse_st = img_lse[y * s.W + x];
         } else if (part == 1) {
-            fetch(kst, a.k, tl, y0, bc, nr, side);
+            fetch(kst, a.k, img_k, y0, bc, nr, side);
         } else if (part == 2) {
-            fetch(vst, a.v, tl, y0, bc, nr, side);
+            fetch(vst, a.v, img_v, y0, bc, nr, side);
         } else if (part == 3) {
-            fetch(gst, a.d_o, tl, y0, bc, nr, side);
+            fetch(gst, a.d_o, img_g, y0, bc, nr, side);
         } else {
-            fetch(ost, a.o, tl, y0, bc, nr, side);
+            fetch(ost, a.o, img_o, y0, bc, nr, side);
         }
     };
     // registers -> LDS; image row y goes to row slot (y + HALF) % HR
-    auto commit = [&](int y0, auto nr) __attribute__((always_inline)) {
+    auto commit_as = [&](int y0, auto nr, auto side) __attribute__((always_inline)) {
         constexpr int NR = decltype(nr)::value;
+        constexpr int SIDE = decltype(side)::value;
+        constexpr int MINE = SIDE == 0 ? F::q_passes(NR) : F::passes(NR) - F::q_passes(NR);
         const int s0 = (y0 + HALF) % G::HR;
         auto lds_row = [&](int pr, int pc) __attribute__((always_inline)) {
             int slot = s0 + pr;
@@ -243,9 +253,9 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
             return slot * G::HC + pc;
         };
 #pragma unroll
-        for (int i = 0; i < F::q_passes(NR); i++) {
+        for (int i = 0; i < MINE; i++) {
             const float d = group_sum<G::CPR>(dot8<BF>(gst.v[i], ost.v[i]));
-            const int pix = step_pixel(i, nr, role);
+            const int pix = step_pixel(i, nr, SIDE);
             if (pix >= 0) {
                 const int row = lds_row(pix / G::HC, pix % G::HC);
                 const int e = G::chunk_at(row, stid % G::CPR);
@@ -258,17 +268,23 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         }
         if (stid < NR * G::HC) lds_stat[lds_row(stid / G::HC, stid % G::HC)].x = lse_st * kLog2e;
     };
-    // NR rows at once, not overlapped with anything (first tile of a workgroup, first
-    // tile of a column)
     constexpr std::integral_constant<int, 0> kQuerySide{};
     constexpr std::integral_constant<int, 1> kKeySide{};
-    auto stage_now = [&](const Tile &tl, int y0, int bc, auto nr) __attribute__((always_inline)) {
+    // (the side is a per-wave value: a scalar branch, and each side only forms dO . O of
+    // the chunks it staged)
+    auto commit = [&](int y0, auto nr) __attribute__((always_inline)) {
+        if (role == 0) commit_as(y0, nr, kQuerySide);
+        else commit_as(y0, nr, kKeySide);
+    };
+    // NR rows at once, not overlapped with anything (first tile of a workgroup, first
+    // tile of a column)
+    auto stage_now = [&](int y0, int bc, auto nr) __attribute__((always_inline)) {
         if (role == 0) {
 #pragma unroll
-            for (int part = 0; part < 5; part++) fetch_part(tl, part, y0, bc, nr, kQuerySide);
+            for (int part = 0; part < 5; part++) fetch_part(part, y0, bc, nr, kQuerySide);
         } else {
 #pragma unroll
-            for (int part = 0; part < 5; part++) fetch_part(tl, part, y0, bc, nr, kKeySide);
+            for (int part = 0; part < 5; part++) fetch_part(part, y0, bc, nr, kKeySide);
         }
         commit(y0, nr);
     };
@@ -276,8 +292,9 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     constexpr std::integral_constant<int, G::HR - F::BR> kRest{};
 
     Tile cur = tile_of_cm(sc.t, ts.tiles_r, ts.tiles_c, s.N);
-    stage_now(cur, cur.r0 - HALF, cur.c0 - HALF, kStep);
-    stage_now(cur, cur.r0 - HALF + F::BR, cur.c0 - HALF, kRest);
+    set_image(cur);
+    stage_now(cur.r0 - HALF, cur.c0 - HALF, kStep);
+    stage_now(cur.r0 - HALF + F::BR, cur.c0 - HALF, kRest);
     __syncthreads();
     const int n = l & 15, g = l >> 4;
     static_assert(G::SWC == 8 && G::SW == 8 && G::NK == G::NKP,
@@ -304,11 +321,12 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         // the tile below in the same image: its block shares k-1 rows with this one
         const bool below = more && nxt.bb == cur.bb && nxt.nn == cur.nn && nxt.c0 == cur.c0 &&
                            nxt.r0 == cur.r0 + 8;
+        if (nxt.bb != cur.bb || nxt.nn != cur.nn) set_image(nxt);
         const int ny0 = below ? cur.r0 - HALF + G::HR : nxt.r0 - HALF;
         const int nbc = nxt.c0 - HALF;
         auto issue_as = [&](int part, auto side) __attribute__((always_inline)) {
             __builtin_amdgcn_sched_barrier(0);
-            if (more) fetch_part(nxt, part, ny0, nbc, kStep, side);
+            if (more) fetch_part(part, ny0, nbc, kStep, side);
             __builtin_amdgcn_sched_barrier(0);
         };
 
@@ -430,9 +448,9 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
 #pragma unroll
                     for (int mt = 0; mt < G::MT; mt++) {
                         if (mt < 4) issue(mt);
+                        f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
                         const int row = tok_row(2 * mt, n >> 3, ocol + (n & 7));
                         const typename G::ARow qp = G::a_row(lds_q, row, g), gp = G::a_row(lds_g, row, g);
-                        f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int ds = 0; ds < G::DS; ds++) {
                             cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(qp, ds)), kreg[ds], cs);
@@ -479,32 +497,45 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 // ---- key side of a tile beside the border.  The clamped windows make the
                 // set of queries that attend to the wave's 4x4 keys wider, up to SW + k/2
                 // per axis, and the relation depends on where a query's window starts:
-                // walk a (SW + k/2)^2 region, numbered 16 per row, 32 queries at a time,
-                // with one bit per region row / column telling whether that query row /
-                // column attends this lane's key row / column.  The loop is rolled
+                // walk that region 32 queries at a time, with one bit per region row /
+                // column telling whether that query row / column attends this lane's key
+                // row / column.  The loop is rolled
                 // (unrolled, the addresses of the whole region would be formed up front).
                 const int ky0 = cur.r0 + (w >> 1) * 4, kx0 = cur.c0 + (w & 1) * 4;
-                constexpr int side = F::SWB;  // region side
-                constexpr int nks = F::KSB;   // reduction steps of 32 queries
-                const int orow = min(max(inv_lo(ky0, KS) - br, 0), G::HR - F::SWB);
-                const int ocol = min(max(inv_lo(kx0, KS) - bc, 0), G::HC - F::SWB);
+                // query rows / columns that attend the wave's key rows / columns: SW of them
+                // away from the border, SW - k/2 or SW + k/2 beside it
+                const int qr0 = inv_lo(ky0, KS), qc0 = inv_lo(kx0, KS);
+                const int nr = inv_hi(ky0 + 3, s.H, KS) - qr0, nc = inv_hi(kx0 + 3, s.W, KS) - qc0;
+                const int orow = qr0 - br, ocol = qc0 - bc;
+                // The region is numbered along its shorter side where that has at most SW
+                // queries (8 per line, else 16), so that its lines fill the 32-query steps:
+                // 2 or 3 steps for a wave beside one border, 5 only in a corner.
+                const bool tr = nc > G::SW && nr <= G::SW;  // lines are columns
+                const int nmaj = tr ? nc : nr, nmin = tr ? nr : nc;
+                const int lsh = nmin > G::SW ? 4 : 3;
+                const int nks = ((nmaj << lsh) + 31) >> 5;
                 unsigned rmask = 0, cmask = 0;
 #pragma unroll
                 for (int r = 0; r < F::SWB; r++) {
-                    const int qy = br + orow + r, qx = bc + ocol + r;
-                    const bool oky = (r < side) & ((unsigned)qy < (unsigned)s.H) &
-                                     ((unsigned)(py - win_start(qy, s.H, KS)) < (unsigned)KS);
-                    const bool okx = (r < side) & ((unsigned)qx < (unsigned)s.W) &
-                                     ((unsigned)(px - win_start(qx, s.W, KS)) < (unsigned)KS);
+                    const int qy = qr0 + r, qx = qc0 + r;
+                    const bool oky = (r < nr) & ((unsigned)(py - win_start(qy, s.H, KS)) < (unsigned)KS);
+                    const bool okx = (r < nc) & ((unsigned)(px - win_start(qx, s.W, KS)) < (unsigned)KS);
                     rmask |= (oky ? 1u : 0u) << r;
                     cmask |= (okx ? 1u : 0u) << r;
                 }
-                // region (row, column) of query number tk
-                auto reg_r = [&](int tk) __attribute__((always_inline)) { return tk >> 4; };
-                auto reg_c = [&](int tk) __attribute__((always_inline)) { return tk & 15; };
+                // region (row, column) of query number tk; numbers beyond the region have
+                // a row or column whose mask bit is clear
+                auto reg_r = [&](int tk) __attribute__((always_inline)) {
+                    const int maj = tk >> lsh, mn = tk & ((1 << lsh) - 1);
+                    return tr ? mn : maj;
+                };
+                auto reg_c = [&](int tk) __attribute__((always_inline)) {
+                    const int maj = tk >> lsh, mn = tk & ((1 << lsh) - 1);
+                    return tr ? maj : mn;
+                };
                 auto row_of = [&](int tk) __attribute__((always_inline)) {
                     const int r = reg_r(tk), c = reg_c(tk);
-                    return ((r < side) & (c < side)) ? block_row(orow + r, ocol + c) : (int)G::ZROW;
+                    return ((r < nr) & (c < nc)) ? block_row(orow + r, ocol + c) : (int)G::ZROW;
                 };
                 auto ok_of = [&](int tk) __attribute__((always_inline)) {
                     return ((rmask >> reg_r(tk)) & (cmask >> reg_c(tk)) & 1u) != 0u;
@@ -581,7 +612,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         if (!more) break;
         __syncthreads();  // every wave is done with this tile's LDS
         commit(ny0, kStep);
-        if (!below) stage_now(nxt, ny0 + F::BR, nbc, kRest);
+        if (!below) stage_now(ny0 + F::BR, nbc, kRest);
         __syncthreads();
         cur = nxt;
         sc.t = tn;
