@@ -336,7 +336,7 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, co
     a.zinv = a.delta + (size_t)B * heads * T;
     a.s = Shape{B, heads, 1, T, D, 1, kernel_size, scale};
     if (g_path.load() != ENATTEN_PATH_SIMT && mfma1d_supported(D, kernel_size, dtype))
-        return launch_bwd1d_mfma(a, dtype, static_cast<hipStream_t>(stream));
+        return launch_bwd1d_mfma(a, dtype, g_path.load(), static_cast<hipStream_t>(stream));
     return launch_bwd_simt(a, dtype, static_cast<hipStream_t>(stream));
 }
 

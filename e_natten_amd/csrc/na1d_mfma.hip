@@ -457,6 +457,203 @@ __global__ __launch_bounds__(256, 2) void bwd1d_dkdv_mfma(BwdArgs a, int tiles_t
     }
 }
 
+// ------------------------------------------------------------------ dQ, dK, dV in one pass
+// The rows of q, k, v and dO that a tile of 64 positions needs, as queries' keys and as
+// keys' queries, are staged ONCE: positions [row0, row0 + RQ), where row0 is the smaller of
+// the window start of the tile's first query and the first query that attends its first
+// key.  delta = dO . O of every staged query is formed while the rows are written to LDS
+// (the forward output is read for this and for nothing else), so the backward reads five
+// tensors and writes three where the two passes read eight and write three.  Each wave
+// first forms dQ of its 16 positions (as bwd1d_dq_mfma), then dK and dV of the same 16
+// positions (as bwd1d_dkdv_mfma), all operands out of LDS.
+// Workgroups per CU that the registers are budgeted for: what LDS admits, at most three.
+// (At head_dim 128 LDS holds one workgroup; a variant with eight waves there, four for dQ
+// and four for dK and dV, was measured level with this one.)
+template <bool BF, int D, int NKP>
+__global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fused_mfma(
+    BwdArgs a, int tiles_t, int ntiles) {
+    using G = Geo1<D, NKP>;
+    constexpr int NR = G::RQ, CPR = D / 8;
+    __shared__ __attribute__((aligned(16))) short lds_q[(NR + 1) * G::PITCH];
+    __shared__ __attribute__((aligned(16))) short lds_g[(NR + 1) * G::PITCH];
+    __shared__ __attribute__((aligned(16))) short lds_k[(NR + 1) * G::PITCH];
+    __shared__ __attribute__((aligned(16))) short lds_v[(NR + 1) * G::PITCH];
+    __shared__ float2 lds_stat[NR + 1];  // (lse * log2e, dO . O) per staged position
+    const Shape &s = a.s;
+    const int T = s.W, ks = s.kw;
+    Sched sc = make_sched(ntiles, blockIdx.x, gridDim.x);
+    if (sc.t >= sc.t_end) return;
+    zero_row1<D>(lds_q, NR);
+    zero_row1<D>(lds_g, NR);
+    zero_row1<D>(lds_k, NR);
+    zero_row1<D>(lds_v, NR);
+    if (threadIdx.x == 0) lds_stat[NR] = make_float2(0.f, 0.f);
+    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const float sc2 = s.scale * kLog2e;
+    const int ntok = 15 + ks;
+
+    using St = Stage1<D, NR>;
+    St qst, gst, kst, vst, ost;
+    float lse_st = 0.f;
+    static_assert(NR <= 256, "one log-sum-exp per thread");
+    auto row0_of = [&](const Tile1 &tl) __attribute__((always_inline)) {
+        return min(win_start(tl.t0, T, ks), inv_lo(tl.t0, ks));
+    };
+    auto prefetch = [&](const Tile1 &tl) __attribute__((always_inline)) {
+        const int ra = row0_of(tl);
+        qst.fetch(seq(a.q, tl), a.q.sw, ra, T);
+        kst.fetch(seq(a.k, tl), a.k.sw, ra, T);
+        vst.fetch(seq(a.v, tl), a.v.sw, ra, T);
+        gst.fetch(seq(a.d_o, tl), a.d_o.sw, ra, T);
+        ost.fetch(seq(a.o, tl), a.o.sw, ra, T);
+        const int64_t sq0 = ((int64_t)tl.bb * s.N + tl.nn) * T;
+        lse_st = a.lse[sq0 + min(ra + min((int)threadIdx.x, NR - 1), T - 1)];
+    };
+    Tile1 cur = tile1_of(sc.t, tiles_t, s.N);
+    prefetch(cur);
+    for (;;) {
+        qst.commit(lds_q);
+        gst.commit(lds_g);
+        kst.commit(lds_k);
+        vst.commit(lds_v);
+#pragma unroll
+        for (int i = 0; i < St::NL; i++) {
+            const float d = group_sum<CPR>(dot8<BF>(gst.v[i], ost.v[i]));
+            const int r = (int)threadIdx.x / CPR + i * St::RPP;
+            if (r < NR && threadIdx.x % CPR == 0) lds_stat[r].y = d;
+        }
+        if (threadIdx.x < NR) lds_stat[threadIdx.x].x = lse_st * kLog2e;
+        __syncthreads();
+        const int tn = sc.t + sc.step;
+        const bool more = tn < sc.t_end;
+        Tile1 nxt = cur;
+        if (more) {
+            nxt = tile1_of(tn, tiles_t, s.N);
+            prefetch(nxt);
+        }
+        const int ra = row0_of(cur);
+        const int w0 = cur.t0 + wave * 16;
+        if (w0 < T) {
+            const bool live = w0 + n < T;
+            const int pt = min(w0 + n, T - 1);  // this lane's position, as query and as key
+            const int64_t tok = ((int64_t)cur.bb * s.N + cur.nn) * T + pt;
+            const int own = pt - ra;
+            {
+                // ---- dQ: the wave's keys are the 16 + k - 1 positions from the window start
+                // of its first query on
+                const int sr0 = win_start(w0, T, ks);
+                const int orow = sr0 - ra, dd = win_start(pt, T, ks) - sr0;
+                auto trow = [&](int tk) __attribute__((always_inline)) {
+                    return tk < ntok ? orow + tk : (int)NR;
+                };
+                s16x8 qreg[G::DS], greg[G::DS];
+#pragma unroll
+                for (int ds = 0; ds < G::DS; ds++) {
+                    qreg[ds] = *reinterpret_cast<const s16x8 *>(lds_q + own * G::PITCH + g * 8 + ds * 32);
+                    greg[ds] = *reinterpret_cast<const s16x8 *>(lds_g + own * G::PITCH + g * 8 + ds * 32);
+                }
+                const float2 mine = lds_stat[own];
+                s16x8 dsb[G::KSTEPS];
+#pragma unroll
+                for (int mt = 0; mt < G::MT; mt++) {
+                    const int row = trow(mt * 16 + n);
+                    const short *kp = lds_k + row * G::PITCH + g * 8, *vp = lds_v + row * G::PITCH + g * 8;
+                    f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ds = 0; ds < G::DS; ds++) {
+                        cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(kp + ds * 32), qreg[ds], cs);
+                        cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(vp + ds * 32), greg[ds], cp);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int tk = mt * 16 + g * 4 + i;
+                        const bool ok = (unsigned)(tk - dd) < (unsigned)ks;
+                        const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - mine.x : -INFINITY);
+                        dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - mine.y));
+                    }
+                }
+                f32x4 dq[G::DT];
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++) dq[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kk = 0; kk < G::KSTEPS; kk++) {
+                    const short *kp[2];
+#pragma unroll
+                    for (int h = 0; h < 2; h++)
+                        kp[h] = lds_k + trow(kk * 32 + h * 16 + g * 4 + (n >> 2)) * G::PITCH + (n & 3) * (D / 4);
+#pragma unroll
+                    for (int mt = 0; mt < G::DT; mt++)
+                        dq[mt] = mfma16<BF>(cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)),
+                                            dsb[kk], dq[mt]);
+                }
+                store_token<BF, D>(static_cast<short *>(a.dq) + tok * D, g, dq, s.scale, live);
+            }
+            {
+                // ---- dK, dV: the queries that attend to any of the wave's 16 keys, 32 at a time
+                s16x8 kreg[G::DS], vreg[G::DS];
+#pragma unroll
+                for (int ds = 0; ds < G::DS; ds++) {
+                    kreg[ds] = *reinterpret_cast<const s16x8 *>(lds_k + own * G::PITCH + g * 8 + ds * 32);
+                    vreg[ds] = *reinterpret_cast<const s16x8 *>(lds_v + own * G::PITCH + g * 8 + ds * 32);
+                }
+                f32x4 dk[G::DT], dv[G::DT];
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++) {
+                    dk[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    dv[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+                const int wa = inv_lo(w0, ks), wb = inv_hi(min(w0 + 16, T) - 1, T, ks);
+                const int nq = wb - wa, r0 = wa - ra;
+                auto row_of = [&](int qi) __attribute__((always_inline)) {
+                    return qi < nq ? r0 + qi : (int)NR;
+                };
+                for (int q0 = 0; q0 < nq; q0 += 32) {
+                    s16x8 pb, dsb;
+#pragma unroll
+                    for (int m2 = 0; m2 < 2; m2++) {
+                        const int row = row_of(q0 + m2 * 16 + n);
+                        const short *qp = lds_q + row * G::PITCH + g * 8, *gp = lds_g + row * G::PITCH + g * 8;
+                        f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int ds = 0; ds < G::DS; ds++) {
+                            cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(qp + ds * 32), kreg[ds], cs);
+                            cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(gp + ds * 32), vreg[ds], cp);
+                        }
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const int qi = q0 + m2 * 16 + g * 4 + i;
+                            const float2 st = lds_stat[row_of(qi)];
+                            const bool ok = (qi < nq) &
+                                            ((unsigned)(pt - win_start(wa + qi, T, ks)) < (unsigned)ks);
+                            const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
+                            pb[m2 * 4 + i] = cvt16<BF>(p);
+                            dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
+                        }
+                    }
+                    const short *qt[2], *gt[2];
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const int row = row_of(q0 + h * 16 + g * 4 + (n >> 2));
+                        qt[h] = lds_q + row * G::PITCH + (n & 3) * (D / 4);
+                        gt[h] = lds_g + row * G::PITCH + (n & 3) * (D / 4);
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < G::DT; mt++) {
+                        dv[mt] = mfma16<BF>(cat(lds_read_tr(gt[0] + mt * 4), lds_read_tr(gt[1] + mt * 4)), pb, dv[mt]);
+                        dk[mt] = mfma16<BF>(cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)), dsb, dk[mt]);
+                    }
+                }
+                store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, live);
+                store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, live);
+            }
+        }
+        if (!more) break;
+        __syncthreads();
+        cur = nxt;
+        sc.t = tn;
+    }
+}
+
 // ------------------------------------------------------------------ dispatch
 template <bool BF, int D, int NKP>
 int fwd1d_launch(const FwdArgs &a, hipStream_t st) {
@@ -468,6 +665,19 @@ int fwd1d_launch(const FwdArgs &a, hipStream_t st) {
         hipLaunchKernelGGL((fwd1d_mfma<BF, D, NKP>), dim3(grid), dim3(256), 0, st, a, tiles_t, (int)nt);
     }
     return check_launch("enatten1d_fwd");
+}
+
+template <bool BF, int D, int NKP>
+int bwd1d_fused_launch(const BwdArgs &a, hipStream_t st) {
+    const int tiles_t = (a.s.W + 63) / 64;
+    const int64_t nt = (int64_t)a.s.B * a.s.N * tiles_t;
+    {
+        ProfScope prof(ENATTEN_KERNEL_BWD_FUSED, "bwd1d_fused_mfma", st);
+        hipLaunchKernelGGL((bwd1d_fused_mfma<BF, D, NKP>),
+                           dim3(persistent_grid<bwd1d_fused_mfma<BF, D, NKP>>(nt)), dim3(256), 0, st, a,
+                           tiles_t, (int)nt);
+    }
+    return check_launch("enatten1d_bwd");
 }
 
 template <bool BF, int D, int NKP>
@@ -526,11 +736,21 @@ int launch_fwd1d_mfma(const FwdArgs &a, int dtype, hipStream_t st) {
     return ENATTEN_EUNSUPPORTED;
 }
 
-int launch_bwd1d_mfma(const BwdArgs &a, int dtype, hipStream_t st) {
+// One-pass backward where it was measured faster than the two passes: every head_dim for
+// kernel_size <= 17, head_dim <= 64 beyond (at head_dim 128 the 136 staged rows of four
+// tensors fill LDS and the two are level).
+bool fused1d_supported(const BwdArgs &a) {
+    return (a.s.kw <= 17 || a.s.D <= 64) && layout1d_ok(a.o);
+}
+
+int launch_bwd1d_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st) {
     auto al = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
     if (!layout1d_ok(a.q) || !layout1d_ok(a.k) || !layout1d_ok(a.v) || !layout1d_ok(a.d_o) ||
         !al(a.dq) || !al(a.dk) || !al(a.dv))
         return launch_bwd_simt(a, dtype, st);
+    if (path != ENATTEN_PATH_MFMA_SPLIT && fused1d_supported(a)) {
+        ENATTEN_1D(bwd1d_fused_launch, a, dtype, st)
+    }
     ENATTEN_1D(bwd1d_launch, a, dtype, st)
     set_error("no matrix-core kernel for head_dim %d, kernel_size %d", a.s.D, a.s.kw);
     return ENATTEN_EUNSUPPORTED;

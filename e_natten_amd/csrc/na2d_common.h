@@ -96,7 +96,7 @@ int launch_bwd_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st);
 // bf16 / f16, D in {32, 64, 128}, odd kernel_size 3 .. 49
 bool mfma1d_supported(int D, int ks, int dtype);
 int launch_fwd1d_mfma(const FwdArgs &a, int dtype, hipStream_t st);
-int launch_bwd1d_mfma(const BwdArgs &a, int dtype, hipStream_t st);
+int launch_bwd1d_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st);
 // fused backward (dQ, dK, dV of every tile from one staging), where built
 bool fused_bwd_supported(const BwdArgs &a);
 int launch_bwd_fused(const BwdArgs &a, bool bf16, const TileSet &ts, int64_t ntiles,

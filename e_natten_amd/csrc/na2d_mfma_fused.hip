@@ -25,8 +25,6 @@
 // The kernel is persistent like the others: the next tile's rows travel from HBM
 // into registers while the current tile is computed out of LDS.
 
-#include <type_traits>
-
 #include "na2d_mfma.h"
 
 namespace enatten {
@@ -60,45 +58,12 @@ struct Chunks {
     u32x4 v[NL];
 };
 
-// dO . O over the 8 channels of one 16-byte chunk, in float32 FMAs.  The halves of
-// a dword are taken apart with integer operations: a bit_cast of a vector element
-// to a 2-vector of 16-bit floats makes this compiler read the chunk's first dword
-// four times (seen in the generated code, and in wrong results).
-template <bool BF>
-__device__ __forceinline__ float half_of(uint32_t w, bool high) {
-    const uint32_t h = high ? w >> 16 : w & 0xffffu;
-    if constexpr (BF) return __uint_as_float(h << 16);
-    else return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
-}
-template <bool BF>
-__device__ __forceinline__ float dot8(u32x4 a, u32x4 b) {
-    float even = 0.f, odd = 0.f;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        even = fmaf(half_of<BF>(a[j], false), half_of<BF>(b[j], false), even);
-        odd = fmaf(half_of<BF>(a[j], true), half_of<BF>(b[j], true), odd);
-    }
-    return even + odd;
-}
 // ok ? x : -inf as bit arithmetic.  Written as a conditional expression, the compiler
 // moves the LDS read that feeds x under a branch on ok (one branch per logit).
 __device__ __forceinline__ float keep_or_ninf(float x, bool ok) {
     const int m = ok ? -1 : 0;
     return __int_as_float((__float_as_int(x) & m) | ((int)0xff800000 & ~m));
 }
-// sum over aligned groups of LANES (4, 8 or 16) consecutive lanes, in every lane
-template <int LANES>
-__device__ __forceinline__ float group_sum(float x) {
-    auto step = [&](auto ctrl) __attribute__((always_inline)) {
-        x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), decltype(ctrl)::value, 0xf, 0xf, true));
-    };
-    step(std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]
-    step(std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]
-    if constexpr (LANES >= 8) step(std::integral_constant<int, 0x141>{});   // row_half_mirror
-    if constexpr (LANES >= 16) step(std::integral_constant<int, 0x140>{});  // row_mirror
-    return x;
-}
-
 template <bool BF, int D, int KS>
 __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int ntiles) {
     using G = Geo<D, KS>;

@@ -15,6 +15,14 @@ def _lib():
     return ensure_built()
 
 
+@pytest.fixture(params=["auto", "split"])
+def path(request, _lib):
+    # auto: the one-pass backward where it is built; split: always the dQ and dK/dV passes
+    prev = _lib.enatten_set_path({"auto": 0, "split": 4}[request.param])
+    yield request.param
+    _lib.enatten_set_path(prev)
+
+
 def _run(shape, dtype, ks, seed=0, scale=1.0):
     from e_natten_amd import Natten1d
     g = torch.Generator().manual_seed(seed)
@@ -71,7 +79,7 @@ def test_gradcheck_shape_of_reference():
     ((1, 1, 120, 64), 51, torch.bfloat16),   # beyond them: general kernels
     ((1, 2, 1 << 18, 32), 7, torch.bfloat16),  # a long sequence: 4096 tiles per (batch, head)
 ])
-def test_shapes_1d(shape, ks, dtype):
+def test_shapes_1d(shape, ks, dtype, path):
     _run(shape, dtype, ks, seed=2)
 
 

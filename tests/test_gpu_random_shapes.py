@@ -63,14 +63,23 @@ def _cases_1d(n, seed):
         ks = rnd.choice([3, 5, 7, 9, 13, 17, 19, 25, 33, 49, 51])
         T = rnd.randint(ks, 700)
         B, N = rnd.choice([1, 2, 3]), rnd.choice([1, 2, 5])
-        out.append(((B, N, T, D), ks, dt, it))
+        out.append(((B, N, T, D), ks, dt, it, rnd.choice([0, 4])))
     return out
 
 
-@pytest.mark.parametrize("shape,ks,dtype,seed", _cases_1d(16, 7))
-def test_random_shapes_1d(shape, ks, dtype, seed, lib):
+@pytest.mark.parametrize("shape,ks,dtype,seed,path", _cases_1d(24, 7))
+def test_random_shapes_1d(shape, ks, dtype, seed, path, lib):
     from e_natten_amd import Natten1d
-    print("case random 1d", shape, "k=%d" % ks, dtype, flush=True)
+    print("case random 1d", shape, "k=%d" % ks, dtype, "path", path, flush=True)
+    prev = lib.enatten_set_path(path)  # 0: one-pass backward where built, 4: two passes
+    try:
+        _random_1d(shape, ks, dtype, seed)
+    finally:
+        lib.enatten_set_path(prev)
+
+
+def _random_1d(shape, ks, dtype, seed):
+    from e_natten_amd import Natten1d
     g = torch.Generator().manual_seed(200 + seed)
     q, k, v, d_o = (torch.randn(shape, generator=g).to(dtype) for _ in range(4))
     ref = O1.natten1d_explicit(q, k, v, d_o, ks)
