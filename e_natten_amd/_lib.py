@@ -8,7 +8,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libenatten.so")
 
-ABI_VERSION = 3  # ENATTEN_ABI_VERSION of include/enatten.h
+ABI_VERSION = 4  # ENATTEN_ABI_VERSION of include/enatten.h
 F32, BF16, F16 = 0, 1, 2
 STATIC_BWD_MAX_QUERIES = 1 << 20
 PATH_NONE, PATH_SIMT, PATH_MFMA, PATH_MFMA_FUSED, PATH_MFMA_SPLIT = 0, 1, 2, 3, 4
@@ -30,6 +30,9 @@ SIGNATURES = {
     "enatten2d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 7),
     "enatten2d_bwd": (_i, [_vp] * 10 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
     "enatten2d_bwd_static": (_i, [_vp] * 9 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
+    "enatten2d_fwd_window": (_i, [_vp] * 5 + [_i] * 10 + [_sp] * 4 + [ctypes.c_float, _vp]),
+    "enatten2d_bwd_window_workspace_bytes": (ctypes.c_size_t, [_i] * 4),
+    "enatten2d_bwd_window": (_i, [_vp] * 10 + [_i] * 10 + [_sp] * 5 + [ctypes.c_float, _vp]),
     "enatten1d_fwd": (_i, [_vp] * 5 + [_i] * 6 + [_sp] * 4 + [ctypes.c_float, _vp]),
     "enatten1d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 3),
     "enatten1d_bwd": (_i, [_vp] * 10 + [_i] * 6 + [_sp] * 5 + [ctypes.c_float, _vp]),

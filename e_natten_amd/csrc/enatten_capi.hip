@@ -255,6 +255,90 @@ int enatten2d_bwd_static(const void *q, const void *k, const void *v, const void
                  q_strides, k_strides, v_strides, o_strides, do_strides, scale, stream);
 }
 
+// ---- rectangular and causal windows ----------------------------------------
+// One axis of a window: extent k, causal or centred.
+static int check_axis(const char *fn, const char *axis, int L, int k, int causal) {
+    if (k < 1 || (!causal && k % 2 == 0)) {
+        set_error("%s: kernel_%s must be >= 1, and odd unless that axis is causal, got %d", fn,
+                  axis, k);
+        return ENATTEN_EINVAL;
+    }
+    if (L < k) {
+        set_error("%s: the image has %d positions along %s, fewer than kernel_%s = %d", fn, L, axis,
+                  axis, k);
+        return ENATTEN_EINVAL;
+    }
+    return ENATTEN_OK;
+}
+
+int enatten2d_fwd_window(const void *q, const void *k, const void *v, void *o, float *lse, int B,
+                         int heads, int H, int W, int D, int kernel_h, int kernel_w, int causal_h,
+                         int causal_w, int dtype, const int64_t *q_strides,
+                         const int64_t *k_strides, const int64_t *v_strides,
+                         const int64_t *o_strides, float scale, void *stream) {
+    if (kernel_h == kernel_w && !causal_h && !causal_w)
+        return enatten2d_fwd(q, k, v, o, lse, B, heads, H, W, D, kernel_h, dtype, q_strides,
+                             k_strides, v_strides, o_strides, scale, stream);
+    const char *fn = "enatten2d_fwd_window";
+    int rc = check_shape(fn, B, heads, H, W, D, 1, dtype);
+    if (rc) return rc;
+    if ((rc = check_axis(fn, "h", H, kernel_h, causal_h))) return rc;
+    if ((rc = check_axis(fn, "w", W, kernel_w, causal_w))) return rc;
+    FwdArgs a;
+    if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
+    if ((rc = make_view(fn, "k", k, k_strides, heads, H, W, D, &a.k))) return rc;
+    if ((rc = make_view(fn, "v", v, v_strides, heads, H, W, D, &a.v))) return rc;
+    if ((rc = make_view(fn, "o", o, o_strides, heads, H, W, D, &a.o))) return rc;
+    a.lse = lse;
+    a.s = Shape{B, heads, H, W, D, kernel_h, kernel_w, scale, causal_h ? 1 : 0, causal_w ? 1 : 0};
+    return launch_fwd_simt(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+size_t enatten2d_bwd_window_workspace_bytes(int B, int heads, int H, int W) {
+    if (B < 1 || heads < 1 || H < 1 || W < 1) return 0;
+    return (size_t)B * heads * H * W * 2 * sizeof(float);
+}
+
+int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void *o,
+                         const void *d_o, const float *lse, void *dq, void *dk, void *dv,
+                         void *workspace, int B, int heads, int H, int W, int D, int kernel_h,
+                         int kernel_w, int causal_h, int causal_w, int dtype,
+                         const int64_t *q_strides, const int64_t *k_strides,
+                         const int64_t *v_strides, const int64_t *o_strides,
+                         const int64_t *do_strides, float scale, void *stream) {
+    const char *fn = "enatten2d_bwd_window";
+    const bool plain = kernel_h == kernel_w && !causal_h && !causal_w;
+    int rc = check_shape(fn, B, heads, H, W, D, plain ? kernel_h : 1, dtype);
+    if (rc) return rc;
+    if (!workspace) {
+        set_error("%s: workspace is NULL", fn);
+        return ENATTEN_EINVAL;
+    }
+    const size_t ws_floats = (size_t)B * heads * H * W * 2;
+    if (plain)  // the reference's window: every kernel family that two floats per query allow
+        return bwd2d(fn, q, k, v, o, d_o, lse, dq, dk, dv, static_cast<float *>(workspace),
+                     ws_floats, B, heads, H, W, D, kernel_h, dtype, q_strides, k_strides, v_strides,
+                     o_strides, do_strides, scale, stream);
+    if ((rc = check_axis(fn, "h", H, kernel_h, causal_h))) return rc;
+    if ((rc = check_axis(fn, "w", W, kernel_w, causal_w))) return rc;
+    BwdArgs a;
+    if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
+    if ((rc = make_view(fn, "k", k, k_strides, heads, H, W, D, &a.k))) return rc;
+    if ((rc = make_view(fn, "v", v, v_strides, heads, H, W, D, &a.v))) return rc;
+    if ((rc = make_view(fn, "o", o, o_strides, heads, H, W, D, &a.o))) return rc;
+    if ((rc = make_view(fn, "d_o", d_o, do_strides, heads, H, W, D, &a.d_o))) return rc;
+    if (!lse || !dq || !dk || !dv) {
+        set_error("%s: lse, dq, dk and dv must all be non-NULL", fn);
+        return ENATTEN_EINVAL;
+    }
+    a.lse = lse;
+    a.dq = dq; a.dk = dk; a.dv = dv;
+    a.delta = static_cast<float *>(workspace);
+    a.zinv = a.delta + (size_t)B * heads * H * W;
+    a.s = Shape{B, heads, H, W, D, kernel_h, kernel_w, scale, causal_h ? 1 : 0, causal_w ? 1 : 0};
+    return launch_bwd_simt(a, dtype, static_cast<hipStream_t>(stream));
+}
+
 static int view_1d(const char *fn, const char *name, const void *p, const int64_t *st, int N,
                    int T, int D, View *out) {
     if (!p) {

@@ -16,8 +16,9 @@ struct View {
 
 struct Shape {
     int B, N, H, W, D;
-    int kh, kw;  // window extent on rows / columns (kh == kw for the 2D operator)
+    int kh, kw;  // window extent on rows / columns (kh == kw for the reference's operator)
     float scale;
+    int ch, cw;  // causal rows / columns: a query only sees keys at or before it on that axis
 };
 
 struct FwdArgs {
@@ -49,6 +50,23 @@ __host__ __device__ inline int win_start(int i, int L, int k) {
 __host__ __device__ inline int inv_lo(int i, int k) { return i < k ? 0 : i - (k >> 1); }
 __host__ __device__ inline int inv_hi(int i, int L, int k) {
     return i >= L - k ? L : i + (k >> 1) + 1;
+}
+
+// The same rules with the causal variant of an axis (NATTEN's causal neighbourhood: the
+// last k positions up to and including the query's own, fewer at the start of the axis;
+// the reference has no causal mode).  A query at i sees keys [axis_start, axis_start +
+// axis_count); a key at j is seen by the queries [axis_inv_lo, axis_inv_hi).
+__host__ __device__ inline int axis_start(int i, int L, int k, int causal) {
+    return causal ? (i - k + 1 < 0 ? 0 : i - k + 1) : win_start(i, L, k);
+}
+__host__ __device__ inline int axis_count(int i, int L, int k, int causal) {
+    return causal ? i - axis_start(i, L, k, 1) + 1 : k;
+}
+__host__ __device__ inline int axis_inv_lo(int j, int k, int causal) {
+    return causal ? j : inv_lo(j, k);
+}
+__host__ __device__ inline int axis_inv_hi(int j, int L, int k, int causal) {
+    return causal ? (j + k < L ? j + k : L) : inv_hi(j, L, k);
 }
 
 // The 8x8 tiles of an image split into an inner rectangle, where no key or query

@@ -156,7 +156,8 @@ template <typename T, int G, int CH, bool VEC>
 __global__ __launch_bounds__(256) void fwd_simt(FwdArgs a, int tiles_x, int tiles_y) {
     const Shape &s = a.s;
     const Place<G> pl(s, tiles_y, tiles_x);
-    const int x0 = win_start(pl.x, s.H, s.kh), y0 = win_start(pl.y, s.W, s.kw);
+    const int x0 = axis_start(pl.x, s.H, s.kh, s.ch), y0 = axis_start(pl.y, s.W, s.kw, s.cw);
+    const int nx = axis_count(pl.x, s.H, s.kh, s.ch), ny = axis_count(pl.y, s.W, s.kw, s.cw);
 
     float qr[CH][8], acc[CH][8];
     const T *qp = at<T>(a.q, pl.b, pl.n, pl.x, pl.y);
@@ -170,8 +171,8 @@ __global__ __launch_bounds__(256) void fwd_simt(FwdArgs a, int tiles_x, int tile
     using A = typename LogitAcc<T>::type;
     A m = -INFINITY;
     float l = 0.f;
-    for (int i = 0; i < s.kh; i++) {
-        for (int j = 0; j < s.kw; j++) {
+    for (int i = 0; i < nx; i++) {
+        for (int j = 0; j < ny; j++) {
             const T *kp = at<T>(a.k, pl.b, pl.n, x0 + i, y0 + j);
             const T *vp = at<T>(a.v, pl.b, pl.n, x0 + i, y0 + j);
             A part = 0;
@@ -218,7 +219,8 @@ template <typename T, int G, int CH, bool VEC>
 __global__ __launch_bounds__(256) void bwd_dq_simt(BwdArgs a, int tiles_x, int tiles_y) {
     const Shape &s = a.s;
     const Place<G> pl(s, tiles_y, tiles_x);
-    const int x0 = win_start(pl.x, s.H, s.kh), y0 = win_start(pl.y, s.W, s.kw);
+    const int x0 = axis_start(pl.x, s.H, s.kh, s.ch), y0 = axis_start(pl.y, s.W, s.kw, s.cw);
+    const int nx = axis_count(pl.x, s.H, s.kh, s.ch), ny = axis_count(pl.y, s.W, s.kw, s.cw);
     const int64_t tok = (((int64_t)pl.b * s.N + pl.n) * s.H + pl.x) * s.W + pl.y;
 
     float qr[CH][8], gr[CH][8], acc[CH][8], pk[CH][8];
@@ -249,8 +251,8 @@ __global__ __launch_bounds__(256) void bwd_dq_simt(BwdArgs a, int tiles_x, int t
     const float delta = group_sum<G>(dpart);
     const A lse = a.lse[tok];
     float zsum = 0.f, esum = 0.f;
-    for (int i = 0; i < s.kh; i++) {
-        for (int j = 0; j < s.kw; j++) {
+    for (int i = 0; i < nx; i++) {
+        for (int j = 0; j < ny; j++) {
             const T *kp = at<T>(a.k, pl.b, pl.n, x0 + i, y0 + j);
             const T *vp = at<T>(a.v, pl.b, pl.n, x0 + i, y0 + j);
             float kr[CH][8];
@@ -305,8 +307,8 @@ template <typename T, int G, int CH, bool VEC>
 __global__ __launch_bounds__(256) void bwd_dkdv_simt(BwdArgs a, int tiles_x, int tiles_y) {
     const Shape &s = a.s;
     const Place<G> pl(s, tiles_y, tiles_x);
-    const int qx0 = inv_lo(pl.x, s.kh), qx1 = inv_hi(pl.x, s.H, s.kh);
-    const int qy0 = inv_lo(pl.y, s.kw), qy1 = inv_hi(pl.y, s.W, s.kw);
+    const int qx0 = axis_inv_lo(pl.x, s.kh, s.ch), qx1 = axis_inv_hi(pl.x, s.H, s.kh, s.ch);
+    const int qy0 = axis_inv_lo(pl.y, s.kw, s.cw), qy1 = axis_inv_hi(pl.y, s.W, s.kw, s.cw);
 
     float kr[CH][8], vr[CH][8], dk[CH][8], dv[CH][8];
     const T *kp = at<T>(a.k, pl.b, pl.n, pl.x, pl.y);

@@ -279,12 +279,126 @@ class Natten2dDilated(torch.autograd.Function):
         return dQ, dK, dV, None, None, None
 
 
-def natten2d(q, k, v, kernel_size=7, scale=1.0, dilation=1):
+def _pair(x, what, kind):
+    """An int / bool or a pair of them -> a pair."""
+    if isinstance(x, (tuple, list)):
+        if len(x) != 2:
+            raise ValueError("%s must have one entry per image axis" % what)
+        x = tuple(x)
+    else:
+        x = (x, x)
+    for e in x:
+        if kind is int and (not isinstance(e, int) or isinstance(e, bool)):
+            raise TypeError("%s must be an int or a pair of ints" % what)
+        if kind is bool and not isinstance(e, (bool, int)):
+            raise TypeError("%s must be a bool or a pair of bools" % what)
+    return x if kind is int else (bool(x[0]), bool(x[1]))
+
+
+def _validate_window(q, k, v, kernel, causal) -> None:
+    _validate(q, k, v, 1)
+    for L, ks, c, axis in zip(q.shape[2:4], kernel, causal, ("rows", "columns")):
+        if ks < 1 or (not c and ks % 2 == 0):
+            raise ValueError("kernel_size along %s must be >= 1, and odd unless that axis is "
+                             "causal, got %d" % (axis, ks))
+        if L < ks:
+            raise ValueError("input has %d %s, fewer than kernel_size %d" % (L, axis, ks))
+
+
+def _window_fwd(q, k, v, kernel, causal, scale: float):
+    _validate_window(q, k, v, kernel, causal)
+    _require_gpu(q, "natten2d")
+    if q.device.type != "cuda":
+        raise RuntimeError("natten2d: rectangular and causal windows need tensors on the GPU")
+    lib = _lib.load()
+    q, k, v = (_kernel_layout(t) for t in (q, k, v))
+    B, N, H, W, D = q.shape
+    with torch.cuda.device(q.device):
+        o = _kernel_layout(torch.empty_like(q))
+        lse = torch.empty((B, N, H, W), dtype=torch.float32, device=q.device)
+        _check(lib.enatten2d_fwd_window(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), B, N, H, W, D,
+            kernel[0], kernel[1], int(causal[0]), int(causal[1]), _DTYPES[q.dtype],
+            _lib.strides4(q), _lib.strides4(k), _lib.strides4(v), _lib.strides4(o), float(scale),
+            _stream_of(q)))
+    return o, lse
+
+
+def _window_bwd(q, k, v, o, lse, d_o, kernel, causal, scale: float):
+    lib = _lib.load()
+    q, k, v, o, d_o = (_kernel_layout(t) for t in (q, k, v, o, d_o))
+    B, N, H, W, D = q.shape
+    with torch.cuda.device(q.device):
+        dq = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
+        dk, dv = torch.empty_like(dq), torch.empty_like(dq)
+        ws = torch.empty(lib.enatten2d_bwd_window_workspace_bytes(B, N, H, W), dtype=torch.uint8,
+                         device=q.device)
+        _check(lib.enatten2d_bwd_window(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(), lse.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, kernel[0],
+            kernel[1], int(causal[0]), int(causal[1]), _DTYPES[q.dtype], _lib.strides4(q),
+            _lib.strides4(k), _lib.strides4(v), _lib.strides4(o), _lib.strides4(d_o), float(scale),
+            _stream_of(q)))
+    return dq, dk, dv
+
+
+class Natten2dWindow(torch.autograd.Function):
+    """2D neighborhood attention with a rectangular and / or causal window (NATTEN's
+    definitions; the reference has one odd kernel_size and no causal mode):
+    ``kernel = (rows, columns)``, ``causal = (rows, columns)``.  On a causal axis a query
+    attends the last k positions up to and including its own.  Served by the general
+    kernels through ``enatten2d_fwd_window`` / ``enatten2d_bwd_window``."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V, kernel, causal, scale):
+        o, lse = _window_fwd(Q, K, V, kernel, causal, scale)
+        ctx.save_for_backward(Q, K, V, o, lse)
+        ctx.args = (kernel, causal, scale)
+        return o
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_output):
+        Q, K, V, o, lse = ctx.saved_tensors
+        dQ, dK, dV = _window_bwd(Q, K, V, o, lse, grad_output, *ctx.args)
+        return dQ, dK, dV, None, None, None
+
+
+def _window_call(q, k, v, kernel, causal, scale, dilation):
+    """Natten2dWindow on the dilation^2 strided sub-grids (see Natten2dDilated)."""
+    if dilation == 1:
+        return Natten2dWindow.apply(q, k, v, kernel, causal, float(scale))
+    if not isinstance(dilation, int) or isinstance(dilation, bool) or dilation < 1:
+        raise ValueError("dilation must be a positive int")
+    _validate_window(q, k, v, kernel, causal)
+    for L, ks in zip(q.shape[2:4], kernel):
+        if L > 1 and L < ks * dilation:
+            raise ValueError("input of extent %d is smaller than kernel_size * dilation = %d"
+                             % (L, ks * dilation))
+    o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    for i in range(dilation if q.shape[2] > 1 else 1):
+        for j in range(dilation):
+            sub = (slice(None), slice(None),
+                   slice(i, None, dilation) if q.shape[2] > 1 else slice(None),
+                   slice(j, None, dilation))
+            o[sub] = Natten2dWindow.apply(q[sub], k[sub], v[sub], kernel, causal, float(scale))
+    return o
+
+
+def natten2d(q, k, v, kernel_size=7, scale=1.0, dilation=1, is_causal=False):
     """``natten2d(q, k, v, kernel_size) -> out`` on ``[B, heads, H, W, d]`` tensors,
     differentiable in q, k and v: the reference's entry point
     (e_natten/triton.py:550, e_natten/__init__.py:1), positional like it.
     ``dilation`` > 1 spaces every neighborhood's keys that far apart (needs image sides
-    of at least kernel_size * dilation)."""
+    of at least kernel_size * dilation).  Beyond the reference, as in NATTEN:
+    ``kernel_size`` may be a pair (rows, columns), and ``is_causal`` (a bool or a pair)
+    makes an axis causal: a query then attends the last kernel_size positions up to and
+    including its own."""
+    if isinstance(kernel_size, (tuple, list)) or is_causal is not False:
+        kernel, causal = _pair(kernel_size, "kernel_size", int), _pair(is_causal, "is_causal", bool)
+        if kernel[0] != kernel[1] or any(causal):
+            return _window_call(q, k, v, kernel, causal, scale, dilation)
+        kernel_size = kernel[0]
     if dilation != 1:
         if not isinstance(dilation, int) or isinstance(dilation, bool) or dilation < 1:
             raise ValueError("dilation must be a positive int")
@@ -352,9 +466,18 @@ class Natten1dDilated(torch.autograd.Function):
         return dQ, dK, dV, None, None, None
 
 
-def natten1d(q, k, v, kernel_size=7, scale=1.0, dilation=1):
+def natten1d(q, k, v, kernel_size=7, scale=1.0, dilation=1, is_causal=False):
     """``natten1d(q, k, v, kernel_size) -> out`` on ``[B, heads, T, d]`` tensors
-    (e_natten/triton.py:485, e_natten/__init__.py:1).  ``dilation`` as in natten2d."""
+    (e_natten/triton.py:485, e_natten/__init__.py:1).  ``dilation`` as in natten2d;
+    ``is_causal=True`` (not in the reference) is sliding-window causal attention: query t
+    attends keys max(t - kernel_size + 1, 0) .. t."""
+    if is_causal:
+        _validate(q, k, v, 1, 4)
+        if not isinstance(kernel_size, int) or isinstance(kernel_size, bool):
+            raise TypeError("kernel_size must be an int")
+        o = _window_call(q.unsqueeze(2), k.unsqueeze(2), v.unsqueeze(2), (1, kernel_size),
+                         (False, True), scale, dilation)
+        return o.squeeze(2)
     if dilation != 1:
         if not isinstance(dilation, int) or isinstance(dilation, bool) or dilation < 1:
             raise ValueError("dilation must be a positive int")

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define ENATTEN_ABI_VERSION 3
+#define ENATTEN_ABI_VERSION 4
 
 /* element types of q, k, v, o and the gradients */
 enum { ENATTEN_F32 = 0, ENATTEN_BF16 = 1, ENATTEN_F16 = 2 };
@@ -136,6 +136,35 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o,
 int enatten2d_bwd_static(const void *q, const void *k, const void *v, const void *o,
                          const void *d_o, const float *lse, void *dq, void *dk, void *dv,
                          int B, int heads, int H, int W, int D, int kernel_size, int dtype,
+                         const int64_t *q_strides, const int64_t *k_strides,
+                         const int64_t *v_strides, const int64_t *o_strides,
+                         const int64_t *do_strides, float scale, void *stream);
+
+/*
+ * Rectangular and causal windows.  They have no counterpart in the reference, which has
+ * one odd kernel_size for both axes and no causal mode (e_natten/triton.py:489,
+ * e_natten/pytorch.py:7-11); they follow NATTEN's definitions and are for callers that
+ * move over from it.  Each axis has its own extent, kernel_h rows by kernel_w columns.
+ * On a causal axis a query at position i attends the keys [max(i - k + 1, 0), i]: the last
+ * k positions up to and including its own, fewer at the start of the axis, and k may be
+ * even there; on the other axes the window is the reference's
+ * clamp(i - k/2, 0, L - k) with k odd.  The same conventions as enatten2d_fwd /
+ * enatten2d_bwd otherwise; the workspace holds two float32 per query
+ * (enatten2d_bwd_window_workspace_bytes).  A 1D causal (sliding-window) attention over
+ * [B, heads, T, D] is the call with H = 1, kernel_h = 1, causal_h = 0.  Square, non-causal
+ * calls are handed to the kernels behind enatten2d_fwd / enatten2d_bwd; every other
+ * window runs on the general kernels.
+ */
+int enatten2d_fwd_window(const void *q, const void *k, const void *v, void *o, float *lse,
+                         int B, int heads, int H, int W, int D, int kernel_h, int kernel_w,
+                         int causal_h, int causal_w, int dtype, const int64_t *q_strides,
+                         const int64_t *k_strides, const int64_t *v_strides,
+                         const int64_t *o_strides, float scale, void *stream);
+size_t enatten2d_bwd_window_workspace_bytes(int B, int heads, int H, int W);
+int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void *o,
+                         const void *d_o, const float *lse, void *dq, void *dk, void *dv,
+                         void *workspace, int B, int heads, int H, int W, int D, int kernel_h,
+                         int kernel_w, int causal_h, int causal_w, int dtype,
                          const int64_t *q_strides, const int64_t *k_strides,
                          const int64_t *v_strides, const int64_t *o_strides,
                          const int64_t *do_strides, float scale, void *stream);

@@ -26,6 +26,9 @@ Pinning status (see tests/test_oracle_*.py):
   dQ, dK, dV                 fp64 autograd of two independent forwards,
                              torch.autograd.gradcheck, sum invariants
   Natten2dLoops              equals the gather oracle
+  axis_window_mask /         (rectangular and causal windows, not in the reference) centred
+  natten2d_window_dense_mask axis = win_start; causal axis with k = L = lower triangle; 1D
+                             causal with k = T = torch's is_causal attention; brute-force rows
 Every function here is pinned by one of those checks.  Two accidental behaviours
 of e_natten/pytorch.py are deliberately NOT restated (they contradict its own
 backward, the Triton kernels and the NATTEN definition): its tile offset rule
@@ -431,6 +434,37 @@ def natten2d_dilated_dense_mask(q, k, v, kernel_size: int, dilation: int, scale:
     if H < kernel_size * dilation or W < kernel_size * dilation:
         raise ValueError("image sides must be >= kernel_size * dilation")
     m = dilated_neighbour_mask(H, W, kernel_size, dilation).to(q.device)
+    o = torch.nn.functional.scaled_dot_product_attention(
+        q.reshape(B, N, H * W, D), k.reshape(B, N, H * W, D), v.reshape(B, N, H * W, D),
+        attn_mask=m, scale=scale)
+    return o.reshape(B, N, H, W, D)
+
+
+def axis_window_mask(L: int, k: int, causal: bool = False) -> torch.Tensor:
+    """[L, L] bool, query (row) attends key (column), for one axis.  Not in the reference
+    (one odd kernel_size, no causal mode); NATTEN's published rules, get_window_start /
+    get_window_end for dilation 1: a centred axis has start = clamp(i - k//2, 0, L - k) and
+    k keys (the reference's rule, e_natten/pytorch.py:7-11); a causal axis has
+    start = max(i - k + 1, 0) and end = i + 1, the last k positions up to the query's own."""
+    if k < 1 or k > L or (not causal and k % 2 == 0):
+        raise ValueError("bad window %d on an axis of %d positions" % (k, L))
+    m = torch.zeros(L, L, dtype=torch.bool)
+    for i in range(L):
+        s0 = max(i - k + 1, 0) if causal else win_start(i, L, k)
+        s1 = i + 1 if causal else s0 + k
+        m[i, s0:s1] = True
+    return m
+
+
+def natten2d_window_dense_mask(q, k, v, kernel, causal=(False, False), scale: float = 1.0):
+    """O of 2D neighborhood attention with a kernel[0] x kernel[1] window and per-axis
+    causal flags, through torch's scaled_dot_product_attention with the dense mask built
+    from axis_window_mask; differentiable.  A [B, N, 1, T, D] input with kernel (1, k) is
+    the 1D operator."""
+    B, N, H, W, D = q.shape
+    mr = axis_window_mask(H, kernel[0], causal[0])
+    mc = axis_window_mask(W, kernel[1], causal[1])
+    m = (mr[:, None, :, None] & mc[None, :, None, :]).reshape(H * W, H * W).to(q.device)
     o = torch.nn.functional.scaled_dot_product_attention(
         q.reshape(B, N, H * W, D), k.reshape(B, N, H * W, D), v.reshape(B, N, H * W, D),
         attn_mask=m, scale=scale)

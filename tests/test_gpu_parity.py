@@ -514,3 +514,54 @@ def test_traced_by_torch_compile(_lib):
     assert torch.equal(out.detach(), ref.detach())
     for a, b in zip(got, gref):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("shape,kernel,causal,dtype", [
+    ((1, 2, 12, 14, 16), (3, 7), (False, False), F32),     # rectangular
+    ((2, 1, 9, 20, 32), (9, 5), (False, False), BF),       # one axis fully covered
+    ((1, 2, 10, 11, 8), (3, 3), (True, False), F32),       # causal rows, centred columns
+    ((1, 1, 13, 9, 64), (4, 5), (True, False), F16),       # an even causal extent
+    ((1, 2, 8, 12, 24), (5, 6), (True, True), F32),        # causal on both axes
+    ((2, 2, 16, 16, 128), (1, 7), (False, False), BF),     # a single row per query
+])
+def test_rectangular_and_causal_windows(shape, kernel, causal, dtype, _lib):
+    # natten2d with kernel_size = (rows, columns) and per-axis is_causal against the dense-mask
+    # oracle (oracle/na2d_oracle.py: axis_window_mask), forward and backward
+    from e_natten_amd import natten2d
+    q, k, v, g = make_inputs(shape, dtype, seed=13)
+    print("case window", shape, dtype, kernel, causal, flush=True)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    o_ref = O.natten2d_window_dense_mask(qr, kr, vr, kernel, causal, 0.5)
+    dq_ref, dk_ref, dv_ref = torch.autograd.grad(o_ref, (qr, kr, vr), g.double())
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = natten2d(qg, kg, vg, kernel, 0.5, 1, causal)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), g.cuda())
+    assert_close(tuple(t.detach().cpu() for t in (o, dq, dk, dv)),
+                 (o_ref.detach(), dq_ref, dk_ref, dv_ref), dtype, "window %s %s" % (kernel, causal))
+
+
+def test_square_pair_takes_the_fast_kernels(_lib):
+    # kernel_size = (k, k) without causal axes is the reference's operator: same kernels, same bits
+    from e_natten_amd import natten2d
+    q, k, v, _ = make_inputs((1, 2, 16, 16, 128), BF, seed=3)
+    q, k, v = (t.cuda() for t in (q, k, v))
+    assert torch.equal(natten2d(q, k, v, (5, 5)), natten2d(q, k, v, 5))
+    assert torch.equal(natten2d(q, k, v, 5, is_causal=(False, False)), natten2d(q, k, v, 5))
+
+
+def test_causal_window_with_dilation(_lib):
+    from e_natten_amd import natten2d
+    shape, kernel, causal, dil = (1, 2, 12, 13, 16), (3, 3), (False, True), 2
+    q, k, v, g = make_inputs(shape, F32, seed=17)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    # oracle: the undilated rule on each of the dilation^2 sub-grids
+    o_ref = torch.empty(shape, dtype=torch.float64)
+    for i in range(dil):
+        for j in range(dil):
+            sub = (slice(None), slice(None), slice(i, None, dil), slice(j, None, dil))
+            o_ref[sub] = O.natten2d_window_dense_mask(qr[sub], kr[sub], vr[sub], kernel, causal)
+    ref = torch.autograd.grad(o_ref, (qr, kr, vr), g.double())
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = natten2d(qg, kg, vg, kernel, 1.0, dil, causal)
+    got = torch.autograd.grad(o, (qg, kg, vg), g.cuda())
+    assert_close(tuple(t.detach().cpu() for t in (o, *got)), (o_ref.detach(), *ref), F32, "dilated causal")

@@ -127,3 +127,28 @@ def test_dilated_1d(shape, ks, dil, dtype):
         x, r = x.detach().cpu(), r.detach()
         err = O.max_abs_err(x, r) if dtype == torch.float32 else O.rel_err(x, r)
         assert err <= (FP32_MAX_ABS if dtype == torch.float32 else BF16_REL), (name, err)
+
+
+@pytest.mark.parametrize("shape,ks,dtype", [((2, 2, 100, 32), 7, torch.float32),
+                                            ((1, 3, 257, 64), 16, torch.bfloat16),
+                                            ((2, 2, 48, 16), 48, torch.float32)])
+def test_causal_1d(shape, ks, dtype):
+    # natten1d(..., is_causal=True): query t attends keys max(t - ks + 1, 0) .. t; against the
+    # dense-mask oracle, and for ks = T against torch's own causal attention
+    from e_natten_amd import natten1d
+    g = torch.Generator().manual_seed(23)
+    q, k, v, d_o = (torch.randn(shape, generator=g).to(dtype) for _ in range(4))
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    o_ref = O.natten2d_window_dense_mask(qr.unsqueeze(2), kr.unsqueeze(2), vr.unsqueeze(2), (1, ks),
+                                         (False, True), 0.25).squeeze(2)
+    ref = (o_ref.detach(), *torch.autograd.grad(o_ref, (qr, kr, vr), d_o.double()))
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = natten1d(qg, kg, vg, ks, 0.25, 1, True)
+    got = (o.detach().cpu(), *(t.cpu() for t in torch.autograd.grad(o, (qg, kg, vg), d_o.cuda())))
+    for name, x, r in zip(("O", "dQ", "dK", "dV"), got, ref):
+        err = O.max_abs_err(x, r) if dtype == torch.float32 else O.rel_err(x, r)
+        print("   causal 1d", shape, dtype, "k=%d" % ks, name, "err %.3e" % err, flush=True)
+        assert err <= (FP32_MAX_ABS if dtype == torch.float32 else BF16_REL), (name, err)
+    if ks == shape[2]:
+        sdpa = torch.nn.functional.scaled_dot_product_attention(qg, kg, vg, is_causal=True, scale=0.25)
+        assert (o - sdpa).abs().max().item() < 1e-4

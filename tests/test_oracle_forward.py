@@ -123,3 +123,48 @@ def test_dilated_window_rule_is_the_plain_rule_on_residue_classes(H, W, ks, dil)
             sub = (slice(None), slice(None), slice(i, None, dil), slice(j, None, dil))
             got[sub] = O.natten2d_gather(q[sub], k[sub], v[sub], ks)
     assert torch.allclose(got, ref, atol=1e-12)
+
+
+def test_axis_window_mask_rules():
+    # centred axis: the reference's rule; causal axis: the last k positions up to the
+    # query's own, which for k = L is the lower triangle of ordinary causal attention
+    for L in (1, 2, 5, 9, 16):
+        for k in range(1, L + 1):
+            mc = O.axis_window_mask(L, k, causal=True)
+            for i in range(L):
+                row = mc[i].nonzero().flatten().tolist()
+                assert row == list(range(max(i - k + 1, 0), i + 1)), (L, k, i, row)
+            if k % 2 == 1:
+                m = O.axis_window_mask(L, k)
+                for i in range(L):
+                    s0 = O.win_start(i, L, k)
+                    assert m[i].nonzero().flatten().tolist() == list(range(s0, s0 + k))
+            else:
+                with pytest.raises(ValueError):
+                    O.axis_window_mask(L, k)
+        assert torch.equal(O.axis_window_mask(L, L, causal=True),
+                           torch.ones(L, L).tril().bool())
+
+
+def test_window_dense_mask_special_cases():
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(2, 2, 7, 9, 4, generator=g, dtype=torch.float64) for _ in range(3))
+    # square centred window: the pinned dense-mask oracle of the reference's operator
+    a = O.natten2d_window_dense_mask(q, k, v, (5, 5), (False, False), 0.7)
+    b = O.natten2d_dense_mask(q, k, v, 5, 0.7)
+    assert torch.allclose(a, b, atol=1e-12)
+    # a rectangular window with one full axis: rows attend all rows, columns their 3 neighbours
+    c = O.natten2d_window_dense_mask(q, k, v, (7, 3))
+    s = torch.einsum("bnxyd,bnuwd->bnxyuw", q, k)
+    keep = O.axis_window_mask(9, 3)[None, None, None, :, None, :].expand_as(s)
+    p = torch.softmax(s.masked_fill(~keep, float("-inf")).flatten(-2), -1).view_as(s)
+    assert torch.allclose(c, torch.einsum("bnxyuw,bnuwd->bnxyd", p, v), atol=1e-12)
+    # 1D causal with the window as long as the sequence: textbook causal attention
+    q1, k1, v1 = (t[:, :, :1] for t in (q, k, v))
+    d = O.natten2d_window_dense_mask(q1, k1, v1, (1, 9), (False, True))
+    ref = torch.nn.functional.scaled_dot_product_attention(q1[:, :, 0], k1[:, :, 0], v1[:, :, 0],
+                                                           is_causal=True, scale=1.0)
+    assert torch.allclose(d[:, :, 0], ref, atol=1e-12)
+    # the first query of a causal axis only sees itself: its output is its own value
+    e = O.natten2d_window_dense_mask(q, k, v, (3, 4), (True, True))
+    assert torch.allclose(e[:, :, 0, 0], v[:, :, 0, 0], atol=1e-12)
