@@ -30,9 +30,9 @@ SIGNATURES = {
     "enatten2d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 7),
     "enatten2d_bwd": (_i, [_vp] * 10 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
     "enatten2d_bwd_static": (_i, [_vp] * 9 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
-    "enatten2d_fwd_window": (_i, [_vp] * 5 + [_i] * 10 + [_sp] * 4 + [ctypes.c_float, _vp]),
+    "enatten2d_fwd_window": (_i, [_vp] * 6 + [_i] * 10 + [_sp] * 4 + [ctypes.c_float, _vp]),
     "enatten2d_bwd_window_workspace_bytes": (ctypes.c_size_t, [_i] * 4),
-    "enatten2d_bwd_window": (_i, [_vp] * 10 + [_i] * 10 + [_sp] * 5 + [ctypes.c_float, _vp]),
+    "enatten2d_bwd_window": (_i, [_vp] * 12 + [_i] * 10 + [_sp] * 5 + [ctypes.c_float, _vp]),
     "enatten1d_fwd": (_i, [_vp] * 5 + [_i] * 6 + [_sp] * 4 + [ctypes.c_float, _vp]),
     "enatten1d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 3),
     "enatten1d_bwd": (_i, [_vp] * 10 + [_i] * 6 + [_sp] * 5 + [ctypes.c_float, _vp]),

@@ -271,12 +271,13 @@ static int check_axis(const char *fn, const char *axis, int L, int k, int causal
     return ENATTEN_OK;
 }
 
-int enatten2d_fwd_window(const void *q, const void *k, const void *v, void *o, float *lse, int B,
-                         int heads, int H, int W, int D, int kernel_h, int kernel_w, int causal_h,
-                         int causal_w, int dtype, const int64_t *q_strides,
-                         const int64_t *k_strides, const int64_t *v_strides,
-                         const int64_t *o_strides, float scale, void *stream) {
-    if (kernel_h == kernel_w && !causal_h && !causal_w)
+int enatten2d_fwd_window(const void *q, const void *k, const void *v, const void *rpb, void *o,
+                         float *lse, int B, int heads, int H, int W, int D, int kernel_h,
+                         int kernel_w, int causal_h, int causal_w, int dtype,
+                         const int64_t *q_strides, const int64_t *k_strides,
+                         const int64_t *v_strides, const int64_t *o_strides, float scale,
+                         void *stream) {
+    if (kernel_h == kernel_w && !causal_h && !causal_w && !rpb)
         return enatten2d_fwd(q, k, v, o, lse, B, heads, H, W, D, kernel_h, dtype, q_strides,
                              k_strides, v_strides, o_strides, scale, stream);
     const char *fn = "enatten2d_fwd_window";
@@ -284,6 +285,10 @@ int enatten2d_fwd_window(const void *q, const void *k, const void *v, void *o, f
     if (rc) return rc;
     if ((rc = check_axis(fn, "h", H, kernel_h, causal_h))) return rc;
     if ((rc = check_axis(fn, "w", W, kernel_w, causal_w))) return rc;
+    if (rpb && (causal_h || causal_w)) {
+        set_error("%s: a relative position bias goes with centred axes only", fn);
+        return ENATTEN_EINVAL;
+    }
     FwdArgs a;
     if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
     if ((rc = make_view(fn, "k", k, k_strides, heads, H, W, D, &a.k))) return rc;
@@ -291,6 +296,7 @@ int enatten2d_fwd_window(const void *q, const void *k, const void *v, void *o, f
     if ((rc = make_view(fn, "o", o, o_strides, heads, H, W, D, &a.o))) return rc;
     a.lse = lse;
     a.s = Shape{B, heads, H, W, D, kernel_h, kernel_w, scale, causal_h ? 1 : 0, causal_w ? 1 : 0};
+    a.rpb = rpb;
     return launch_fwd_simt(a, dtype, static_cast<hipStream_t>(stream));
 }
 
@@ -299,15 +305,15 @@ size_t enatten2d_bwd_window_workspace_bytes(int B, int heads, int H, int W) {
     return (size_t)B * heads * H * W * 2 * sizeof(float);
 }
 
-int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void *o,
-                         const void *d_o, const float *lse, void *dq, void *dk, void *dv,
-                         void *workspace, int B, int heads, int H, int W, int D, int kernel_h,
-                         int kernel_w, int causal_h, int causal_w, int dtype,
+int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void *rpb,
+                         const void *o, const void *d_o, const float *lse, void *dq, void *dk,
+                         void *dv, float *d_rpb, void *workspace, int B, int heads, int H, int W,
+                         int D, int kernel_h, int kernel_w, int causal_h, int causal_w, int dtype,
                          const int64_t *q_strides, const int64_t *k_strides,
                          const int64_t *v_strides, const int64_t *o_strides,
                          const int64_t *do_strides, float scale, void *stream) {
     const char *fn = "enatten2d_bwd_window";
-    const bool plain = kernel_h == kernel_w && !causal_h && !causal_w;
+    const bool plain = kernel_h == kernel_w && !causal_h && !causal_w && !rpb;
     int rc = check_shape(fn, B, heads, H, W, D, plain ? kernel_h : 1, dtype);
     if (rc) return rc;
     if (!workspace) {
@@ -321,6 +327,14 @@ int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void
                      o_strides, do_strides, scale, stream);
     if ((rc = check_axis(fn, "h", H, kernel_h, causal_h))) return rc;
     if ((rc = check_axis(fn, "w", W, kernel_w, causal_w))) return rc;
+    if (rpb && (causal_h || causal_w)) {
+        set_error("%s: a relative position bias goes with centred axes only", fn);
+        return ENATTEN_EINVAL;
+    }
+    if (!rpb != !d_rpb) {
+        set_error("%s: rpb and d_rpb come together", fn);
+        return ENATTEN_EINVAL;
+    }
     BwdArgs a;
     if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
     if ((rc = make_view(fn, "k", k, k_strides, heads, H, W, D, &a.k))) return rc;
@@ -336,6 +350,8 @@ int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void
     a.delta = static_cast<float *>(workspace);
     a.zinv = a.delta + (size_t)B * heads * H * W;
     a.s = Shape{B, heads, H, W, D, kernel_h, kernel_w, scale, causal_h ? 1 : 0, causal_w ? 1 : 0};
+    a.rpb = rpb;
+    a.d_rpb = d_rpb;
     return launch_bwd_simt(a, dtype, static_cast<hipStream_t>(stream));
 }
 

@@ -26,6 +26,7 @@ struct FwdArgs {
     View o;      // written; same kind of strided view as q, k, v
     float *lse;  // contiguous [B, N, H, W] or nullptr
     Shape s;
+    const void *rpb = nullptr;  // relative position bias [N, 2*kh-1, 2*kw-1] in the tensors' type
 };
 
 struct BwdArgs {
@@ -36,6 +37,8 @@ struct BwdArgs {
     float *delta;        // scratch [B, N, H, W]: sum_j P_j dP_j per query
     float *zinv;         // scratch [B, N, H, W]: 1 / sum_j exp(S_j - lse) (vector-ALU kernels)
     Shape s;
+    const void *rpb = nullptr;  // relative position bias [N, 2*kh-1, 2*kw-1] in the tensors' type
+    float *d_rpb = nullptr;     // its gradient, float32, accumulated with atomics (general kernels)
 };
 
 // NATTEN window start on an axis of length L: centred, shifted to stay inside

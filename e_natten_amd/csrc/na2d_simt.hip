@@ -151,6 +151,14 @@ __device__ inline const T *at(const View &v, int b, int n, int x, int y) {
     return static_cast<const T *>(v.ptr) + b * v.sb + n * v.sn + x * v.sh + y * v.sw;
 }
 
+// Relative position bias of (query, key): entry (key - query + k - 1) per axis of the
+// head's [2*kh-1, 2*kw-1] table (NATTEN's rule; the reference has no bias).
+template <typename T>
+__device__ inline float rpb_at(const void *rpb, const Shape &s, int n, int qx, int qy, int kx, int ky) {
+    const int a = kx - qx + s.kh - 1, b = ky - qy + s.kw - 1;
+    return cvt_in(static_cast<const T *>(rpb)[((int64_t)n * (2 * s.kh - 1) + a) * (2 * s.kw - 1) + b]);
+}
+
 // ---------------------------------------------------------------- forward
 template <typename T, int G, int CH, bool VEC>
 __global__ __launch_bounds__(256) void fwd_simt(FwdArgs a, int tiles_x, int tiles_y) {
@@ -184,7 +192,8 @@ __global__ __launch_bounds__(256) void fwd_simt(FwdArgs a, int tiles_x, int tile
 #pragma unroll
                 for (int e = 0; e < 8; e++) part = fma((A)qr[c][e], (A)kr[e], part);
             }
-            const A sc = group_sum<G>(part) * (A)s.scale;
+            A sc = group_sum<G>(part) * (A)s.scale;
+            if (a.rpb) sc += (A)rpb_at<T>(a.rpb, s, pl.n, pl.x, pl.y, x0 + i, y0 + j);
             const A mn = sc > m ? sc : m;
             const float corr = exp_neg(m - mn);
             const float pj = exp_neg(sc - mn);
@@ -270,7 +279,9 @@ __global__ __launch_bounds__(256) void bwd_dq_simt(BwdArgs a, int tiles_x, int t
                     pd = fmaf(gr[c][e], vr[e], pd);
                 }
             }
-            const float p = exp_neg(group_sum<G>(ps) * (A)s.scale - lse);
+            A sl = group_sum<G>(ps) * (A)s.scale;
+            if (a.rpb) sl += (A)rpb_at<T>(a.rpb, s, pl.n, pl.x, pl.y, x0 + i, y0 + j);
+            const float p = exp_neg(sl - lse);
             const float ds = p * (group_sum<G>(pd) - delta);
             zsum += p;
             esum += ds;
@@ -342,9 +353,15 @@ __global__ __launch_bounds__(256) void bwd_dkdv_simt(BwdArgs a, int tiles_x, int
                     pd = fmaf(gr[c][e], vr[c][e], pd);
                 }
             }
-            const float p =
-                exp_neg(group_sum<G>(ps) * (A)s.scale - (A)a.lse[qtok]) * a.zinv[qtok];
+            A sl = group_sum<G>(ps) * (A)s.scale;
+            if (a.rpb) sl += (A)rpb_at<T>(a.rpb, s, pl.n, xi, yi, pl.x, pl.y);
+            const float p = exp_neg(sl - (A)a.lse[qtok]) * a.zinv[qtok];
             const float ds = p * (group_sum<G>(pd) - a.delta[qtok]);
+            // d(bias) of this (query, key) pair is dS itself; here P and dS are final (the
+            // dQ pass left 1 / Z and the corrected delta)
+            if (a.d_rpb && pl.live && pl.lg == 0)
+                atomicAdd(a.d_rpb + ((int64_t)pl.n * (2 * s.kh - 1) + (pl.x - xi + s.kh - 1)) *
+                                        (2 * s.kw - 1) + (pl.y - yi + s.kw - 1), ds);
 #pragma unroll
             for (int c = 0; c < CH; c++)
 #pragma unroll

@@ -305,8 +305,24 @@ def _validate_window(q, k, v, kernel, causal) -> None:
             raise ValueError("input has %d %s, fewer than kernel_size %d" % (L, axis, ks))
 
 
-def _window_fwd(q, k, v, kernel, causal, scale: float):
+def _validate_rpb(q, rpb, kernel, causal) -> None:
+    if not isinstance(rpb, torch.Tensor):
+        raise TypeError("rpb must be a tensor")
+    want = (q.shape[1], 2 * kernel[0] - 1, 2 * kernel[1] - 1)
+    if tuple(rpb.shape) != want:
+        raise ValueError("rpb must have shape [heads, 2*kh-1, 2*kw-1] = %s, got %s"
+                         % (list(want), list(rpb.shape)))
+    if rpb.dtype != q.dtype or rpb.device != q.device:
+        raise ValueError("rpb must have the dtype and device of q")
+    if any(causal):
+        raise ValueError("a relative position bias goes with centred axes only")
+
+
+def _window_fwd(q, k, v, rpb, kernel, causal, scale: float):
     _validate_window(q, k, v, kernel, causal)
+    if rpb is not None:
+        _validate_rpb(q, rpb, kernel, causal)
+        rpb = rpb.contiguous()
     _require_gpu(q, "natten2d")
     if q.device.type != "cuda":
         raise RuntimeError("natten2d: rectangular and causal windows need tensors on the GPU")
@@ -317,57 +333,67 @@ def _window_fwd(q, k, v, kernel, causal, scale: float):
         o = _kernel_layout(torch.empty_like(q))
         lse = torch.empty((B, N, H, W), dtype=torch.float32, device=q.device)
         _check(lib.enatten2d_fwd_window(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), B, N, H, W, D,
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), rpb.data_ptr() if rpb is not None else None,
+            o.data_ptr(), lse.data_ptr(), B, N, H, W, D,
             kernel[0], kernel[1], int(causal[0]), int(causal[1]), _DTYPES[q.dtype],
             _lib.strides4(q), _lib.strides4(k), _lib.strides4(v), _lib.strides4(o), float(scale),
             _stream_of(q)))
     return o, lse
 
 
-def _window_bwd(q, k, v, o, lse, d_o, kernel, causal, scale: float):
+def _window_bwd(q, k, v, rpb, o, lse, d_o, kernel, causal, scale: float):
     lib = _lib.load()
     q, k, v, o, d_o = (_kernel_layout(t) for t in (q, k, v, o, d_o))
     B, N, H, W, D = q.shape
     with torch.cuda.device(q.device):
         dq = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
         dk, dv = torch.empty_like(dq), torch.empty_like(dq)
+        d_rpb = None
+        if rpb is not None:
+            rpb = rpb.contiguous()
+            d_rpb = torch.zeros(rpb.shape, dtype=torch.float32, device=q.device)
         ws = torch.empty(lib.enatten2d_bwd_window_workspace_bytes(B, N, H, W), dtype=torch.uint8,
                          device=q.device)
         _check(lib.enatten2d_bwd_window(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(), lse.data_ptr(),
-            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, kernel[0],
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), rpb.data_ptr() if rpb is not None else None,
+            o.data_ptr(), d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+            dv.data_ptr(), d_rpb.data_ptr() if rpb is not None else None, ws.data_ptr(),
+            B, N, H, W, D, kernel[0],
             kernel[1], int(causal[0]), int(causal[1]), _DTYPES[q.dtype], _lib.strides4(q),
             _lib.strides4(k), _lib.strides4(v), _lib.strides4(o), _lib.strides4(d_o), float(scale),
             _stream_of(q)))
-    return dq, dk, dv
+    return dq, dk, dv, (d_rpb.to(q.dtype) if rpb is not None else None)
 
 
 class Natten2dWindow(torch.autograd.Function):
     """2D neighborhood attention with a rectangular and / or causal window (NATTEN's
     definitions; the reference has one odd kernel_size and no causal mode):
     ``kernel = (rows, columns)``, ``causal = (rows, columns)``.  On a causal axis a query
-    attends the last k positions up to and including its own.  Served by the general
-    kernels through ``enatten2d_fwd_window`` / ``enatten2d_bwd_window``."""
+    attends the last k positions up to and including its own.  ``rpb`` is None or a
+    relative position bias ``[heads, 2*rows-1, 2*columns-1]`` that is added to the scaled
+    logits (entry key - query + kernel - 1 per axis) and gets a gradient.  Served by the
+    general kernels through ``enatten2d_fwd_window`` / ``enatten2d_bwd_window``."""
 
     @staticmethod
-    def forward(ctx, Q, K, V, kernel, causal, scale):
-        o, lse = _window_fwd(Q, K, V, kernel, causal, scale)
-        ctx.save_for_backward(Q, K, V, o, lse)
+    def forward(ctx, Q, K, V, rpb, kernel, causal, scale):
+        o, lse = _window_fwd(Q, K, V, rpb, kernel, causal, scale)
+        ctx.save_for_backward(Q, K, V, o, lse, *(() if rpb is None else (rpb,)))
         ctx.args = (kernel, causal, scale)
         return o
 
     @staticmethod
     @torch.autograd.function.once_differentiable
     def backward(ctx, grad_output):
-        Q, K, V, o, lse = ctx.saved_tensors
-        dQ, dK, dV = _window_bwd(Q, K, V, o, lse, grad_output, *ctx.args)
-        return dQ, dK, dV, None, None, None
+        Q, K, V, o, lse, *rest = ctx.saved_tensors
+        dQ, dK, dV, d_rpb = _window_bwd(Q, K, V, rest[0] if rest else None, o, lse, grad_output,
+                                        *ctx.args)
+        return dQ, dK, dV, d_rpb, None, None, None
 
 
-def _window_call(q, k, v, kernel, causal, scale, dilation):
+def _window_call(q, k, v, kernel, causal, scale, dilation, rpb=None):
     """Natten2dWindow on the dilation^2 strided sub-grids (see Natten2dDilated)."""
     if dilation == 1:
-        return Natten2dWindow.apply(q, k, v, kernel, causal, float(scale))
+        return Natten2dWindow.apply(q, k, v, rpb, kernel, causal, float(scale))
     if not isinstance(dilation, int) or isinstance(dilation, bool) or dilation < 1:
         raise ValueError("dilation must be a positive int")
     _validate_window(q, k, v, kernel, causal)
@@ -381,11 +407,11 @@ def _window_call(q, k, v, kernel, causal, scale, dilation):
             sub = (slice(None), slice(None),
                    slice(i, None, dilation) if q.shape[2] > 1 else slice(None),
                    slice(j, None, dilation))
-            o[sub] = Natten2dWindow.apply(q[sub], k[sub], v[sub], kernel, causal, float(scale))
+            o[sub] = Natten2dWindow.apply(q[sub], k[sub], v[sub], rpb, kernel, causal, float(scale))
     return o
 
 
-def natten2d(q, k, v, kernel_size=7, scale=1.0, dilation=1, is_causal=False):
+def natten2d(q, k, v, kernel_size=7, scale=1.0, dilation=1, is_causal=False, rpb=None):
     """``natten2d(q, k, v, kernel_size) -> out`` on ``[B, heads, H, W, d]`` tensors,
     differentiable in q, k and v: the reference's entry point
     (e_natten/triton.py:550, e_natten/__init__.py:1), positional like it.
@@ -393,11 +419,12 @@ def natten2d(q, k, v, kernel_size=7, scale=1.0, dilation=1, is_causal=False):
     of at least kernel_size * dilation).  Beyond the reference, as in NATTEN:
     ``kernel_size`` may be a pair (rows, columns), and ``is_causal`` (a bool or a pair)
     makes an axis causal: a query then attends the last kernel_size positions up to and
-    including its own."""
-    if isinstance(kernel_size, (tuple, list)) or is_causal is not False:
+    including its own; ``rpb`` is a relative position bias ``[heads, 2*kh-1, 2*kw-1]`` added
+    to the scaled logits (differentiable too)."""
+    if isinstance(kernel_size, (tuple, list)) or is_causal is not False or rpb is not None:
         kernel, causal = _pair(kernel_size, "kernel_size", int), _pair(is_causal, "is_causal", bool)
-        if kernel[0] != kernel[1] or any(causal):
-            return _window_call(q, k, v, kernel, causal, scale, dilation)
+        if kernel[0] != kernel[1] or any(causal) or rpb is not None:
+            return _window_call(q, k, v, kernel, causal, scale, dilation, rpb)
         kernel_size = kernel[0]
     if dilation != 1:
         if not isinstance(dilation, int) or isinstance(dilation, bool) or dilation < 1:
@@ -466,17 +493,21 @@ class Natten1dDilated(torch.autograd.Function):
         return dQ, dK, dV, None, None, None
 
 
-def natten1d(q, k, v, kernel_size=7, scale=1.0, dilation=1, is_causal=False):
+def natten1d(q, k, v, kernel_size=7, scale=1.0, dilation=1, is_causal=False, rpb=None):
     """``natten1d(q, k, v, kernel_size) -> out`` on ``[B, heads, T, d]`` tensors
     (e_natten/triton.py:485, e_natten/__init__.py:1).  ``dilation`` as in natten2d;
     ``is_causal=True`` (not in the reference) is sliding-window causal attention: query t
-    attends keys max(t - kernel_size + 1, 0) .. t."""
-    if is_causal:
+    attends keys max(t - kernel_size + 1, 0) .. t; ``rpb`` is a relative position bias
+    ``[heads, 2*kernel_size-1]``."""
+    if is_causal or rpb is not None:
         _validate(q, k, v, 1, 4)
         if not isinstance(kernel_size, int) or isinstance(kernel_size, bool):
             raise TypeError("kernel_size must be an int")
+        if rpb is not None and (not isinstance(rpb, torch.Tensor) or rpb.dim() != 2):
+            raise ValueError("rpb must be a [heads, 2*kernel_size-1] tensor")
         o = _window_call(q.unsqueeze(2), k.unsqueeze(2), v.unsqueeze(2), (1, kernel_size),
-                         (False, True), scale, dilation)
+                         (False, bool(is_causal)), scale, dilation,
+                         None if rpb is None else rpb.unsqueeze(1))
         return o.squeeze(2)
     if dilation != 1:
         if not isinstance(dilation, int) or isinstance(dilation, bool) or dilation < 1:

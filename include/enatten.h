@@ -141,7 +141,7 @@ int enatten2d_bwd_static(const void *q, const void *k, const void *v, const void
                          const int64_t *do_strides, float scale, void *stream);
 
 /*
- * Rectangular and causal windows.  They have no counterpart in the reference, which has
+ * Rectangular and causal windows, relative position bias.  They have no counterpart in the reference, which has
  * one odd kernel_size for both axes and no causal mode (e_natten/triton.py:489,
  * e_natten/pytorch.py:7-11); they follow NATTEN's definitions and are for callers that
  * move over from it.  Each axis has its own extent, kernel_h rows by kernel_w columns.
@@ -151,20 +151,29 @@ int enatten2d_bwd_static(const void *q, const void *k, const void *v, const void
  * clamp(i - k/2, 0, L - k) with k odd.  The same conventions as enatten2d_fwd /
  * enatten2d_bwd otherwise; the workspace holds two float32 per query
  * (enatten2d_bwd_window_workspace_bytes).  A 1D causal (sliding-window) attention over
- * [B, heads, T, D] is the call with H = 1, kernel_h = 1, causal_h = 0.  Square, non-causal
- * calls are handed to the kernels behind enatten2d_fwd / enatten2d_bwd; every other
- * window runs on the general kernels.
+ * [B, heads, T, D] is the call with H = 1, kernel_h = 1, causal_h = 0.
+ *
+ * rpb, NULL or a relative position bias [heads, 2 * kernel_h - 1, 2 * kernel_w - 1] of the
+ * tensors' element type, contiguous: the logit of (query, key) gets entry
+ * (key - query + kernel - 1) of each axis added after the scaling (NATTEN's rule; centred
+ * axes only).  The backward then adds the bias gradient into d_rpb, float32 of the same
+ * shape, which the caller has set to zero: it is accumulated with float atomics, so its
+ * last bits can differ from run to run (dq, dk and dv stay bit-reproducible).
+ *
+ * Square, non-causal calls without a bias are handed to the kernels behind enatten2d_fwd /
+ * enatten2d_bwd; everything else runs on the general kernels.
  */
-int enatten2d_fwd_window(const void *q, const void *k, const void *v, void *o, float *lse,
-                         int B, int heads, int H, int W, int D, int kernel_h, int kernel_w,
-                         int causal_h, int causal_w, int dtype, const int64_t *q_strides,
-                         const int64_t *k_strides, const int64_t *v_strides,
-                         const int64_t *o_strides, float scale, void *stream);
-size_t enatten2d_bwd_window_workspace_bytes(int B, int heads, int H, int W);
-int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void *o,
-                         const void *d_o, const float *lse, void *dq, void *dk, void *dv,
-                         void *workspace, int B, int heads, int H, int W, int D, int kernel_h,
+int enatten2d_fwd_window(const void *q, const void *k, const void *v, const void *rpb, void *o,
+                         float *lse, int B, int heads, int H, int W, int D, int kernel_h,
                          int kernel_w, int causal_h, int causal_w, int dtype,
+                         const int64_t *q_strides, const int64_t *k_strides,
+                         const int64_t *v_strides, const int64_t *o_strides, float scale,
+                         void *stream);
+size_t enatten2d_bwd_window_workspace_bytes(int B, int heads, int H, int W);
+int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void *rpb,
+                         const void *o, const void *d_o, const float *lse, void *dq, void *dk,
+                         void *dv, float *d_rpb, void *workspace, int B, int heads, int H, int W,
+                         int D, int kernel_h, int kernel_w, int causal_h, int causal_w, int dtype,
                          const int64_t *q_strides, const int64_t *k_strides,
                          const int64_t *v_strides, const int64_t *o_strides,
                          const int64_t *do_strides, float scale, void *stream);

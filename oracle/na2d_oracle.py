@@ -456,15 +456,25 @@ def axis_window_mask(L: int, k: int, causal: bool = False) -> torch.Tensor:
     return m
 
 
-def natten2d_window_dense_mask(q, k, v, kernel, causal=(False, False), scale: float = 1.0):
+def natten2d_window_dense_mask(q, k, v, kernel, causal=(False, False), scale: float = 1.0,
+                               rpb=None):
     """O of 2D neighborhood attention with a kernel[0] x kernel[1] window and per-axis
     causal flags, through torch's scaled_dot_product_attention with the dense mask built
     from axis_window_mask; differentiable.  A [B, N, 1, T, D] input with kernel (1, k) is
-    the 1D operator."""
+    the 1D operator.  rpb [N, 2*kh-1, 2*kw-1], if given, is NATTEN's relative position
+    bias: the logit of (query, key) gets rpb[n, key_row - query_row + kh - 1,
+    key_col - query_col + kw - 1] added after the scaling."""
     B, N, H, W, D = q.shape
     mr = axis_window_mask(H, kernel[0], causal[0])
     mc = axis_window_mask(W, kernel[1], causal[1])
     m = (mr[:, None, :, None] & mc[None, :, None, :]).reshape(H * W, H * W).to(q.device)
+    if rpb is not None:
+        ar = (torch.arange(H)[None, :] - torch.arange(H)[:, None] + kernel[0] - 1)  # [query, key]
+        ac = (torch.arange(W)[None, :] - torch.arange(W)[:, None] + kernel[1] - 1)
+        ar = ar.clamp(0, 2 * kernel[0] - 2)[:, None, :, None].expand(H, W, H, W)
+        ac = ac.clamp(0, 2 * kernel[1] - 2)[None, :, None, :].expand(H, W, H, W)
+        bias = rpb[:, ar.reshape(H * W, H * W), ac.reshape(H * W, H * W)]  # [N, HW, HW]
+        m = torch.where(m[None], bias, torch.full_like(bias, float("-inf")))[None]
     o = torch.nn.functional.scaled_dot_product_attention(
         q.reshape(B, N, H * W, D), k.reshape(B, N, H * W, D), v.reshape(B, N, H * W, D),
         attn_mask=m, scale=scale)

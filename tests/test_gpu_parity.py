@@ -565,3 +565,36 @@ def test_causal_window_with_dilation(_lib):
     o = natten2d(qg, kg, vg, kernel, 1.0, dil, causal)
     got = torch.autograd.grad(o, (qg, kg, vg), g.cuda())
     assert_close(tuple(t.detach().cpu() for t in (o, *got)), (o_ref.detach(), *ref), F32, "dilated causal")
+
+
+@pytest.mark.parametrize("shape,kernel,dtype,dil", [
+    ((2, 3, 10, 12, 16), (3, 3), F32, 1),
+    ((1, 2, 9, 14, 32), (5, 3), BF, 1),
+    ((1, 2, 16, 16, 128), (5, 5), F16, 1),     # a square window with a bias: general kernels
+    ((1, 2, 13, 12, 8), (3, 3), F32, 2),       # with dilation: the bias gradient sums over sub-grids
+])
+def test_relative_position_bias(shape, kernel, dtype, dil, _lib):
+    # natten2d(..., rpb=...) against the dense-mask oracle with the bias in the mask; O, dQ,
+    # dK, dV and the bias gradient (accumulated with float atomics: compared, not bit-checked)
+    from e_natten_amd import natten2d
+    q, k, v, g = make_inputs(shape, dtype, seed=19)
+    gen = torch.Generator().manual_seed(3)
+    rpb = torch.randn(shape[1], 2 * kernel[0] - 1, 2 * kernel[1] - 1, generator=gen).to(dtype)
+    print("case rpb", shape, dtype, kernel, "dilation", dil, flush=True)
+    qr, kr, vr, br = (t.double().requires_grad_(True) for t in (q, k, v, rpb))
+    o_ref = torch.empty(shape, dtype=torch.float64)
+    for i in range(dil):
+        for j in range(dil):
+            sub = (slice(None), slice(None), slice(i, None, dil), slice(j, None, dil))
+            o_ref[sub] = O.natten2d_window_dense_mask(qr[sub], kr[sub], vr[sub], kernel, scale=0.4, rpb=br)
+    ref = torch.autograd.grad(o_ref, (qr, kr, vr, br), g.double())
+    qg, kg, vg, bg = (t.cuda().requires_grad_(True) for t in (q, k, v, rpb))
+    o = natten2d(qg, kg, vg, kernel, 0.4, dil, False, bg)
+    got = torch.autograd.grad(o, (qg, kg, vg, bg), g.cuda())
+    assert_close(tuple(t.detach().cpu() for t in (o, *got[:3])), (o_ref.detach(), *ref[:3]), dtype, "rpb")
+    d_rpb, d_ref = got[3].detach().cpu(), ref[3]
+    assert d_rpb.shape == rpb.shape and d_rpb.dtype == dtype
+    err = (O.max_abs_err(d_rpb, d_ref) / max(1.0, d_ref.abs().max().item()) if dtype == F32
+           else O.rel_err(d_rpb, d_ref))
+    print("   d_rpb err %.3e" % err, flush=True)
+    assert err <= (1e-4 if dtype == F32 else BF16_REL)

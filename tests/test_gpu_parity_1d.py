@@ -152,3 +152,22 @@ def test_causal_1d(shape, ks, dtype):
     if ks == shape[2]:
         sdpa = torch.nn.functional.scaled_dot_product_attention(qg, kg, vg, is_causal=True, scale=0.25)
         assert (o - sdpa).abs().max().item() < 1e-4
+
+
+def test_rpb_1d():
+    from e_natten_amd import natten1d
+    g = torch.Generator().manual_seed(29)
+    shape, ks = (2, 3, 77, 16), 7
+    q, k, v, d_o = (torch.randn(shape, generator=g) for _ in range(4))
+    rpb = torch.randn(3, 2 * ks - 1, generator=g)
+    qr, kr, vr, br = (t.double().requires_grad_(True) for t in (q, k, v, rpb))
+    o_ref = O.natten2d_window_dense_mask(qr.unsqueeze(2), kr.unsqueeze(2), vr.unsqueeze(2), (1, ks),
+                                         rpb=br.unsqueeze(1)).squeeze(2)
+    ref = (o_ref.detach(), *torch.autograd.grad(o_ref, (qr, kr, vr, br), d_o.double()))
+    qg, kg, vg, bg = (t.cuda().requires_grad_(True) for t in (q, k, v, rpb))
+    o = natten1d(qg, kg, vg, ks, rpb=bg)
+    got = (o.detach().cpu(), *(t.cpu() for t in torch.autograd.grad(o, (qg, kg, vg, bg), d_o.cuda())))
+    for name, x, r in zip(("O", "dQ", "dK", "dV", "dRPB"), got, ref):
+        err = O.max_abs_err(x, r) / max(1.0, r.abs().max().item())
+        print("   rpb 1d", name, "err %.3e" % err, flush=True)
+        assert err <= FP32_MAX_ABS, (name, err)

@@ -203,17 +203,21 @@ def test_meta_tensors_give_shapes_without_a_gpu():
 
 def test_window_entry_points_validate(lib):
     from e_natten_amd import _lib, natten1d, natten2d
-    f = lambda kh, kw, ch=0, cw=0, H=8, W=8, q=1: lib.enatten2d_fwd_window(
-        q, 1, 1, 1, None, 1, 1, H, W, 16, kh, kw, ch, cw, 0, None, None, None, None, 1.0, None)
+    f = lambda kh, kw, ch=0, cw=0, H=8, W=8, q=1, rpb=None: lib.enatten2d_fwd_window(
+        q, 1, 1, rpb, 1, None, 1, 1, H, W, 16, kh, kw, ch, cw, 0, None, None, None, None, 1.0, None)
     assert f(3, 4) == 1 and "odd unless that axis is causal" in _lib.last_error()
     assert f(9, 3) == 1 and "fewer than kernel_h" in _lib.last_error()
     assert f(3, 0, 0, 1) == 1
     assert f(3, 4, 0, 1, q=None) == 1 and "q is NULL" in _lib.last_error()   # even is fine when causal
     assert f(4, 4) == 1 and "odd" in _lib.last_error()   # square non-causal: the plain entry point's rule
     assert lib.enatten2d_bwd_window_workspace_bytes(2, 3, 4, 5) == 2 * 3 * 4 * 5 * 8
-    assert lib.enatten2d_bwd_window(1, 1, 1, 1, 1, None, 1, 1, 1, None, 1, 1, 8, 8, 16, 3, 5, 0, 0, 0,
-                                    None, None, None, None, None, 1.0, None) == 1
+    assert f(3, 5, 0, 1, rpb=1) == 1 and "centred axes only" in _lib.last_error()
+    assert lib.enatten2d_bwd_window(1, 1, 1, None, 1, 1, None, 1, 1, 1, None, None, 1, 1, 8, 8, 16, 3, 5,
+                                    0, 0, 0, None, None, None, None, None, 1.0, None) == 1
     assert "workspace is NULL" in _lib.last_error()
+    assert lib.enatten2d_bwd_window(1, 1, 1, 1, 1, 1, None, 1, 1, 1, None, 1, 1, 1, 8, 8, 16, 3, 5,
+                                    0, 0, 0, None, None, None, None, None, 1.0, None) == 1
+    assert "rpb and d_rpb come together" in _lib.last_error()
     q = torch.randn(1, 2, 8, 8, 16)
     with pytest.raises(ValueError, match="odd unless"):
         natten2d(q, q, q, (3, 4))
@@ -229,3 +233,9 @@ def test_window_entry_points_validate(lib):
         natten1d(q[0], q[0], q[0], 4, is_causal=True)
     with pytest.raises(ValueError):
         natten1d(q[0], q[0], q[0], 9, is_causal=True)
+    with pytest.raises(ValueError, match="rpb must have shape"):
+        natten2d(q, q, q, 3, rpb=torch.zeros(2, 5, 7))
+    with pytest.raises(ValueError, match="centred axes only"):
+        natten2d(q, q, q, 3, is_causal=(True, False), rpb=torch.zeros(2, 5, 5))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        natten2d(q, q, q, 3, rpb=torch.zeros(2, 5, 5))

@@ -168,3 +168,41 @@ def test_window_dense_mask_special_cases():
     # the first query of a causal axis only sees itself: its output is its own value
     e = O.natten2d_window_dense_mask(q, k, v, (3, 4), (True, True))
     assert torch.allclose(e[:, :, 0, 0], v[:, :, 0, 0], atol=1e-12)
+
+
+def test_relative_position_bias_oracle():
+    # NATTEN's published bias index (get_pb_start: ns + max(ns - i, 0) + min(L - i - 1 - ns, 0),
+    # plus the position inside the window) is key - query + k - 1 for every query of every axis
+    for L in (5, 8, 13):
+        for k in (1, 3, 5):
+            ns = k // 2
+            for i in range(L):
+                pb = ns + (ns - i if i < ns else 0) + (L - i - 1 - ns if i + ns >= L else 0)
+                s0 = O.win_start(i, L, k)
+                for j in range(k):
+                    assert pb + j == (s0 + j) - i + k - 1, (L, k, i, j)
+    g = torch.Generator().manual_seed(9)
+    q, k, v = (torch.randn(1, 2, 6, 7, 4, generator=g, dtype=torch.float64) for _ in range(3))
+    rpb = torch.randn(2, 5, 9, generator=g, dtype=torch.float64, requires_grad=True)
+    base = O.natten2d_window_dense_mask(q, k, v, (3, 5), scale=0.6)
+    # a zero bias and a constant bias change nothing (softmax is shift-invariant)
+    assert torch.allclose(O.natten2d_window_dense_mask(q, k, v, (3, 5), scale=0.6,
+                                                       rpb=torch.zeros(2, 5, 9, dtype=torch.float64)), base)
+    assert torch.allclose(O.natten2d_window_dense_mask(q, k, v, (3, 5), scale=0.6,
+                                                       rpb=torch.full((2, 5, 9), 1.7, dtype=torch.float64)), base)
+    # brute force for one interior and one border query
+    o = O.natten2d_window_dense_mask(q, k, v, (3, 5), scale=0.6, rpb=rpb)
+    for (x, y) in ((3, 3), (0, 6), (5, 0)):
+        x0, y0 = O.win_start(x, 6, 3), O.win_start(y, 7, 5)
+        for n in range(2):
+            logits, vals = [], []
+            for i in range(3):
+                for j in range(5):
+                    kx, ky = x0 + i, y0 + j
+                    logits.append(0.6 * (q[0, n, x, y] @ k[0, n, kx, ky]) + rpb[n, kx - x + 2, ky - y + 4])
+                    vals.append(v[0, n, kx, ky])
+            p = torch.softmax(torch.stack(logits), 0)
+            assert torch.allclose(o[0, n, x, y], (p[:, None] * torch.stack(vals)).sum(0), atol=1e-12)
+    # every query's dS sums to zero, so the bias gradient sums to zero per head
+    (d_rpb,) = torch.autograd.grad((o * torch.randn(o.shape, generator=g, dtype=torch.float64)).sum(), rpb)
+    assert d_rpb.sum((1, 2)).abs().max() < 1e-10 and d_rpb.abs().max() > 1e-3
