@@ -595,25 +595,29 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
     }
 }
 
-// Frame tiles: the general case, walked block by block (see above).
-template <bool BF, int D, int KS, int SP>
+// Frame tiles: the general case, walked block by block (see above).  KSG sets the size of a
+// staged block, (8 + KSG - 1)^2 queries: KS, or more (kFrameKS) so that the queries of a
+// tile in the second ring from the border, up to 16 + k/2 rows and columns of them, are
+// one block instead of up to four.  `lds_red` then lies over the staged rows (RED_OVER):
+// the partial sums are exchanged when a tile's last block has been read by every wave.
+template <bool BF, int D, int KS, int SP, int KSG, bool RED_OVER>
 __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, int ntiles,
                                            int block, int nblocks, short *lds_q, short *lds_g,
                                            float2 *lds_stat, f32x4 *lds_red) {
-    using G = Geo<D, KS, 4, SP>;
+    using G = Geo<D, KSG, 4, SP>;
     const Shape &s = a.s;
     Sched sc = make_sched(ntiles, block, nblocks);
     if (sc.t >= sc.t_end) return;
-    zero_row<D, KS, 4, SP>(lds_q);
-    zero_row<D, KS, 4, SP>(lds_g);
+    zero_row<D, KSG, 4, SP>(lds_q);
+    zero_row<D, KSG, 4, SP>(lds_g);
 
     // wave = block of 4x4 keys (0..3) + 4 * (its part of the block's queries)
     const int wave = (threadIdx.x >> 6) & 3, part = threadIdx.x >> 8;
     const int l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
 
-    const HaloPlan<D, KS, 4, SP> plan = make_plan<D, KS, 4, SP>();
-    HaloRegs<D, KS, 4, SP> qst, gst;
+    const HaloPlan<D, KSG, 4, SP> plan = make_plan<D, KSG, 4, SP>();
+    HaloRegs<D, KSG, 4, SP> qst, gst;
     float2 sst[G::NST];
     // the wave's 4x4 keys of a tile: this lane's key pixel (clamped into the image)
     auto key_of = [&](const Tile &tl, int &kr, int &kc) __attribute__((always_inline)) {
@@ -622,8 +626,8 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
     };
     auto stage = [&](const KeyBlock &b) __attribute__((always_inline)) {
         const int64_t img_tok = ((int64_t)b.tl.bb * s.N + b.tl.nn) * s.H * (int64_t)s.W;
-        halo_fetch<D, KS>(qst, plan, image<short>(a.q, b.tl), a.q.sh, a.q.sw, b.br, b.bc, b.qb, b.cb);
-        halo_fetch<D, KS>(gst, plan, image<short>(a.d_o, b.tl), a.d_o.sh, a.d_o.sw, b.br, b.bc, b.qb, b.cb);
+        halo_fetch<D, KSG>(qst, plan, image<short>(a.q, b.tl), a.q.sh, a.q.sw, b.br, b.bc, b.qb, b.cb);
+        halo_fetch<D, KSG>(gst, plan, image<short>(a.d_o, b.tl), a.d_o.sh, a.d_o.sw, b.br, b.bc, b.qb, b.cb);
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
             const int id = threadIdx.x + i * G::NT;
@@ -670,8 +674,8 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
     stage(cur);
     load_keys(cur.tl);
     for (;;) {
-        halo_commit<D, KS>(lds_q, plan, qst);
-        halo_commit<D, KS>(lds_g, plan, gst);
+        halo_commit<D, KSG>(lds_q, plan, qst);
+        halo_commit<D, KSG>(lds_g, plan, gst);
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
             const int id = threadIdx.x + i * G::NT;
@@ -778,6 +782,7 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
         } else {
             // the second part's sums reach the first through LDS (see dkdv_inner)
             f32x4 *red = lds_red + wave * 64 + l;
+            if (RED_OVER && cur.last) __syncthreads();  // every wave has read the block
             if (cur.last && part == 1) {
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++) {
@@ -796,6 +801,7 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
                 store();
             }
             if (!more) break;
+            if (RED_OVER && cur.last) __syncthreads();  // the sums are read: the next block may land
         }
         cur = nxt;
     }
@@ -810,6 +816,10 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 // three workgroups per CU (head_dim <= 64 with small halos; it fits 168 registers there,
 // measured 35 -> 32 us at B8 N2 112x112 d32 k7 and 67 -> 60 us at B4 N4 128x128 d32 k9;
 // the forward and the dQ pass spill under that budget and get slower).
+// Size of the frame body's blocks as a kernel size (see dkdv_frame): larger than KS where the
+// pass has one workgroup per CU anyway (two parts per block) and LDS has the room.
+template <int D, int KS, int SP>
+constexpr int kFrameKS = SP == 2 && KS >= 9 ? 9 + KS / 2 : KS;
 template <int D, int KS, int SP>
 constexpr int kDkdvWaves =
     SP == 1 && D <= 64 && 3 * (Geo<D, KS>::LDS_BYTES + 2048) <= 160 * 1024 ? 3 : Geo<D, KS, 4, SP>::WAVES;
@@ -817,21 +827,42 @@ template <bool BF, int D, int KS, bool ROLL, int SP = 1>
 __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) void bwd_dkdv_mfma(
     BwdArgs a, TileSet ts, int n_inner, int n_frame, int inner_blocks, Runs rp) {
     using G = Geo<D, KS, 4, SP>;
-    __shared__ __attribute__((aligned(16))) short lds_q[G::ROWS * G::PITCH];
-    __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
-    __shared__ float2 lds_stat[G::ROWS];  // (lse * log2e, delta) per staged query
-    // partial dK and dV of the second part of every block
-    __shared__ f32x4 lds_red[SP > 1 ? 2 * G::DT * 256 : 1];
+    using FG = Geo<D, kFrameKS<D, KS, SP>, 4, SP>;  // blocks of the frame body
+    // One LDS buffer, laid out by each body for itself: staged Q rows, staged dO rows,
+    // (lse * log2e, delta) per staged query, and with two parts per block the second part's
+    // partial dK and dV.  Where the frame body stages larger blocks, its partial sums lie
+    // over its Q rows.
+    constexpr bool RED_OVER = !std::is_same<FG, G>::value;
+    constexpr size_t RED = SP > 1 ? (size_t)2 * G::DT * 256 * sizeof(f32x4) : 0;
+    constexpr size_t I_ROWS = (size_t)G::ROWS * G::PITCH * sizeof(short);
+    constexpr size_t F_ROWS = (size_t)FG::ROWS * FG::PITCH * sizeof(short);
+    constexpr size_t I_STAT = (G::ROWS * sizeof(float2) + 15) / 16 * 16;
+    constexpr size_t F_STAT = (FG::ROWS * sizeof(float2) + 15) / 16 * 16;
+    constexpr size_t I_ALL = 2 * I_ROWS + I_STAT + RED;
+    constexpr size_t F_ALL = 2 * F_ROWS + F_STAT + (RED_OVER ? 0 : RED);
+    static_assert(RED <= F_ROWS || !RED_OVER, "the partial sums lie over the staged Q rows");
+    __shared__ __attribute__((aligned(16))) char lds_raw[I_ALL > F_ALL ? I_ALL : F_ALL];
+    static_assert(sizeof(lds_raw) <= 160 * 1024, "LDS");
     if ((int)blockIdx.x < inner_blocks) {
+        short *lds_q = reinterpret_cast<short *>(lds_raw);
+        short *lds_g = reinterpret_cast<short *>(lds_raw + I_ROWS);
+        float2 *lds_stat = reinterpret_cast<float2 *>(lds_raw + 2 * I_ROWS);
+        f32x4 *lds_red = reinterpret_cast<f32x4 *>(lds_raw + 2 * I_ROWS + I_STAT);
         if (SP == 1 || threadIdx.x < 256)
             dkdv_inner<BF, D, KS, ROLL, SP, 0>(a, ts, n_inner, rp, blockIdx.x, inner_blocks, lds_q,
                                                lds_g, lds_stat, lds_red);
         else  // the same number of barriers as the first part
             dkdv_inner<BF, D, KS, ROLL, SP, SP - 1>(a, ts, n_inner, rp, blockIdx.x, inner_blocks,
                                                     lds_q, lds_g, lds_stat, lds_red);
-    } else
-        dkdv_frame<BF, D, KS, SP>(a, ts, n_frame, blockIdx.x - inner_blocks,
-                                  gridDim.x - inner_blocks, lds_q, lds_g, lds_stat, lds_red);
+    } else {
+        short *lds_q = reinterpret_cast<short *>(lds_raw);
+        short *lds_g = reinterpret_cast<short *>(lds_raw + F_ROWS);
+        float2 *lds_stat = reinterpret_cast<float2 *>(lds_raw + 2 * F_ROWS);
+        f32x4 *lds_red = reinterpret_cast<f32x4 *>(RED_OVER ? lds_raw : lds_raw + 2 * F_ROWS + F_STAT);
+        dkdv_frame<BF, D, KS, SP, kFrameKS<D, KS, SP>, RED_OVER>(
+            a, ts, n_frame, blockIdx.x - inner_blocks, gridDim.x - inner_blocks, lds_q, lds_g,
+            lds_stat, lds_red);
+    }
 }
 
 // ------------------------------------------------------------------ dispatch
@@ -968,7 +999,9 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             // of a frame tile in inner tiles: about 2 when the inner tiles are bound
             // by arithmetic (d <= 64), about 1.15 when they are bound by HBM (d = 128).
             constexpr int SP = kDkdvSplit<D, KS>, NT = Geo<D, KS, 4, SP>::NT;
-            const double cost = D >= 128 ? 1.15 : 2.0;
+            // (1.68 with the frame body's larger blocks: every weight from 1.6 to 1.75 gives the
+            // same split at 128x128)
+            const double cost = D >= 128 ? 1.15 : kFrameKS<D, KS, SP> != KS ? 1.68 : 2.0;
             const int grid = persistent_grid<bwd_dkdv_mfma<BF, D, KS, false, SP>>(nb, NT);
             int inner_blocks = 0;
             if (n_frame == 0) {
