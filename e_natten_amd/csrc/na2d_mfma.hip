@@ -351,6 +351,143 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
     }
 }
 
+// ------------------------------------------------------------------ dQ, one halo in LDS at a time
+// The dQ pass for halos of which LDS holds two only once per CU (head_dim 64 with
+// kernel_size 13): a tile is done in two phases over ONE LDS
+// buffer, so that two workgroups share a CU and each SIMD has two independent waves.
+//   phase 1  V rows in LDS: dP^T = V dO^T for the wave's whole halo, kept in registers;
+//            the tile's K rows are in flight meanwhile and replace V behind a barrier;
+//   phase 2  K rows in LDS: P from the saved log-sum-exp, delta, dS, dQ^T = K^T dS^T;
+//            the next tile's V rows are in flight meanwhile.
+// Four barriers per tile instead of two; 8x8 tiles, no column walk.
+template <bool BF, int D, int KS>
+__global__ __launch_bounds__(256, 2) void bwd_dq2_mfma(BwdArgs a, TileSet ts, int ntiles) {
+    using G = Geo<D, KS>;
+    __shared__ __attribute__((aligned(16))) short lds_x[G::ROWS * G::PITCH];
+    const Shape &s = a.s;
+    Sched sc = make_sched(ntiles, blockIdx.x, gridDim.x);
+    if (sc.t >= sc.t_end) return;
+    zero_row<D, KS>(lds_x);  // (a commit only writes the halo's own rows)
+
+    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const float sc2 = s.scale * kLog2e;
+    const HaloPlan<D, KS> plan = make_plan<D, KS>();
+    HaloRegs<D, KS> st;
+    // This lane's dO row is loaded a phase ahead of phase 1, its q row and log-sum-exp a
+    // phase ahead of phase 2: one spare set of row registers instead of two.
+    s16x8 qreg[G::DS], gnext[G::DS];
+    float lse_cur = 0.f;
+    auto fetch_rows = [&](const View &vw, const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
+        halo_fetch<D, KS>(st, plan, image<short>(vw, tl), vw.sh, vw.sw, lq.hr0, lq.hc0, s.H, s.W);
+    };
+    auto fetch_do = [&](const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
+        const short *gp = image<short>(a.d_o, tl) + lq.qr * a.d_o.sh + lq.qc * a.d_o.sw + g * 8;
+#pragma unroll
+        for (int ds = 0; ds < G::DS; ds++) gnext[ds] = *reinterpret_cast<const s16x8 *>(gp + ds * 32);
+    };
+    auto fetch_q = [&](const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
+        const short *qp = image<short>(a.q, tl) + lq.qr * a.q.sh + lq.qc * a.q.sw + g * 8;
+#pragma unroll
+        for (int ds = 0; ds < G::DS; ds++) qreg[ds] = *reinterpret_cast<const s16x8 *>(qp + ds * 32);
+        lse_cur = a.lse[lq.tok];
+    };
+
+    Tile cur = tile_of(sc.t, ts.tiles_r, ts.tiles_c, s.N);
+    LaneQ lq = lane_query<KS>(cur, s, wave, n);
+    fetch_rows(a.v, cur, lq);
+    fetch_do(cur, lq);
+    for (;;) {
+        halo_commit<D, KS>(lds_x, plan, st);  // V
+        s16x8 greg[G::DS];
+#pragma unroll
+        for (int ds = 0; ds < G::DS; ds++) greg[ds] = gnext[ds];
+        __syncthreads();
+        fetch_rows(a.k, cur, lq);
+        fetch_q(cur, lq);
+        auto trow = [&](int tk) __attribute__((always_inline)) { return G::token_row(tk, lq.orow, lq.ocol); };
+
+        f32x4 dp[G::MT];
+        if (lq.wave_on) {
+#pragma unroll
+            for (int mt = 0; mt < G::MT; mt++) {
+                const typename G::ARow vp = G::a_row(lds_x, trow(mt * 16 + n), g);
+                f32x4 cp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ds = 0; ds < G::DS; ds++)
+                    cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(vp, ds)), greg[ds], cp);
+                dp[mt] = cp;
+            }
+        }
+        __syncthreads();                      // every wave has read V
+        halo_commit<D, KS>(lds_x, plan, st);  // K
+        __syncthreads();
+
+        const int tn = sched_peek(sc);
+        const bool more = tn < sc.t_end;
+        Tile nxt = cur;
+        LaneQ lqn = lq;
+        if (more) {
+            nxt = tile_of(tn, ts.tiles_r, ts.tiles_c, s.N);
+            lqn = lane_query<KS>(nxt, s, wave, n);
+            fetch_rows(a.v, nxt, lqn);
+            fetch_do(nxt, lqn);
+        }
+        const float lse2 = lse_cur * kLog2e;
+        if (lq.wave_on) {
+            s16x8 dsb[G::KSTEPS];
+            float dpart = 0.f;
+#pragma unroll
+            for (int mt = 0; mt < G::MT; mt++) {
+                const typename G::ARow kp = G::a_row(lds_x, trow(mt * 16 + n), g);
+                f32x4 cs = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ds = 0; ds < G::DS; ds++)
+                    cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(kp, ds)), qreg[ds], cs);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int tk = mt * 16 + g * 4 + i;
+                    const int kr = tk / G::SWC, kc = tk % G::SWC;
+                    const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
+                                    (unsigned)(kc - lq.dc) < (unsigned)KS;
+                    const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - lse2 : -INFINITY);
+                    dpart = fmaf(p, dp[mt][i], dpart);
+                    dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p);
+                }
+            }
+            const float delta = col_sum(dpart);
+#pragma unroll
+            for (int mt = 0; mt < G::MT; mt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float p = cvt32<BF>(dsb[mt >> 1][(mt & 1) * 4 + i]);
+                    dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (dp[mt][i] - delta));
+                }
+            f32x4 dq[G::DT];
+#pragma unroll
+            for (int mt = 0; mt < G::DT; mt++) dq[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < G::KSTEPS; ks++) {
+                typename G::TRow kp[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                    kp[h] = G::t_row(lds_x, trow(ks * 32 + h * 16 + g * 4 + (n >> 2)), n);
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++)
+                    dq[mt] = mfma16<BF>(
+                        cat(lds_read_tr(G::t_at(kp[0], mt)), lds_read_tr(G::t_at(kp[1], mt))), dsb[ks],
+                        dq[mt]);
+            }
+            store_token<BF, D>(static_cast<short *>(a.dq) + lq.tok * D, g, dq, s.scale, lq.live);
+            if (lq.live && g == 0) a.delta[lq.tok] = delta;
+        }
+        if (!more) break;
+        __syncthreads();  // every wave has read K
+        cur = nxt;
+        lq = lqn;
+        sched_advance(sc, tn);
+    }
+}
+
 // ------------------------------------------------------------------ dK, dV
 // Key-centric: the workgroup owns an 8x8 tile of keys and stages Q, dO, the
 // log-sum-exp and delta of the queries that attend to them, i.e. the union of the
@@ -898,6 +1035,15 @@ constexpr bool kTallBuilt =
 template <int D, int KS>
 constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= 11;
 
+// The dQ pass with one halo in LDS at a time (bwd_dq2_mfma): where two halos leave LDS for
+// one workgroup per CU, one halo fits twice, and the 16x8 tiles are not used.  head_dim 64
+// (kernel_size 13): 96 -> 79 us at B2 N8 128x128.  At head_dim 128 (kernel_size 7 and 9) it
+// needs more registers than a wave has at two per SIMD (40-50 spilled) and was measured
+// slower (112 -> 162 us, 125 -> 155 us), so it is not built there.
+template <int D, int KS>
+constexpr bool kDq2Built = D == 64 && Geo<D, KS>::WAVES == 1 && !kTallDqBuilt<D, KS> &&
+                           2 * (Geo<D, KS>::ROWS * Geo<D, KS>::PITCH * 2 + 1024) <= 160 * 1024;
+
 // The dK/dV pass with two waves per 4x4 block of keys, each on half of the block's
 // queries (Geo's SP): where the staged queries leave LDS for one workgroup per CU, a
 // SIMD then still holds two waves.  Built for head_dim 64 (the partial sums of the
@@ -971,7 +1117,12 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         }
 
         bool dq_done = false;
-        if constexpr (kTallDqBuilt<D, KS>) {
+        if constexpr (kDq2Built<D, KS>) {
+            const int grid = persistent_grid<bwd_dq2_mfma<BF, D, KS>>(nb);
+            ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq2_mfma", st);
+            hipLaunchKernelGGL((bwd_dq2_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, ts, (int)nb);
+            dq_done = true;
+        } else if constexpr (kTallDqBuilt<D, KS>) {
             using G8 = Geo<D, KS, 8>;
             TileSet tall = ts;  // only the tile counts are used by this pass
             tall.tiles_r = (a.s.H + G8::TH - 1) / G8::TH;
