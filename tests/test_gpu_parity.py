@@ -137,6 +137,10 @@ def test_config5_backbone_stages(heads, side, path):
     ((1, 1, 13, 13, 64), 13, BF),
     ((1, 2, 37, 29, 64), 13, BF),    # two waves per block of keys in the dK/dV pass, ragged sides
     ((2, 1, 43, 52, 64), 11, F16),
+    ((1, 2, 16, 61, 64), 13, BF),    # 22-row frame blocks with a short axis; one-halo dQ pass
+    ((1, 1, 56, 24, 64), 13, F16),   # inner tiles on one axis only
+    ((1, 1, 64, 72, 64), 13, BF),    # inner tiles, second ring and border together
+    ((1, 2, 48, 41, 64), 11, BF),
     ((2, 2, 12, 12, 32), 1, BF),     # k = 1: O == V
     ((1, 2, 20, 18, 64), 5, F16),
     ((1, 2, 20, 18, 128), 7, F16),
