@@ -207,7 +207,15 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         }
     };
     // registers -> LDS; image row y goes to row slot (y + HALF) % HR
-    auto commit_as = [&](int y0, auto nr, auto side) __attribute__((always_inline)) {
+    // dO . O of the chunks this thread staged (every lane of a pixel gets the pixel's sum)
+    auto deltas_as = [&](float (&d)[F::NL], auto nr, auto side) __attribute__((always_inline)) {
+        constexpr int NR = decltype(nr)::value;
+        constexpr int SIDE = decltype(side)::value;
+        constexpr int MINE = SIDE == 0 ? F::q_passes(NR) : F::passes(NR) - F::q_passes(NR);
+#pragma unroll
+        for (int i = 0; i < MINE; i++) d[i] = group_sum<G::CPR>(dot8<BF>(gst.v[i], ost.v[i]));
+    };
+    auto commit_as = [&](int y0, auto nr, auto side, const float (&dl)[F::NL]) __attribute__((always_inline)) {
         constexpr int NR = decltype(nr)::value;
         constexpr int SIDE = decltype(side)::value;
         constexpr int MINE = SIDE == 0 ? F::q_passes(NR) : F::passes(NR) - F::q_passes(NR);
@@ -219,7 +227,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         };
 #pragma unroll
         for (int i = 0; i < MINE; i++) {
-            const float d = group_sum<G::CPR>(dot8<BF>(gst.v[i], ost.v[i]));
+            const float d = dl[i];
             const int pix = step_pixel(i, nr, SIDE);
             if (pix >= 0) {
                 const int row = lds_row(pix / G::HC, pix % G::HC);
@@ -237,9 +245,13 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     constexpr std::integral_constant<int, 1> kKeySide{};
     // (the side is a per-wave value: a scalar branch, and each side only forms dO . O of
     // the chunks it staged)
-    auto commit = [&](int y0, auto nr) __attribute__((always_inline)) {
-        if (role == 0) commit_as(y0, nr, kQuerySide);
-        else commit_as(y0, nr, kKeySide);
+    auto deltas = [&](float (&d)[F::NL], auto nr) __attribute__((always_inline)) {
+        if (role == 0) deltas_as(d, nr, kQuerySide);
+        else deltas_as(d, nr, kKeySide);
+    };
+    auto commit = [&](int y0, auto nr, const float (&d)[F::NL]) __attribute__((always_inline)) {
+        if (role == 0) commit_as(y0, nr, kQuerySide, d);
+        else commit_as(y0, nr, kKeySide, d);
     };
     // NR rows at once, not overlapped with anything (first tile of a workgroup, first
     // tile of a column)
@@ -251,7 +263,9 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
 #pragma unroll
             for (int part = 0; part < 5; part++) fetch_part(part, y0, bc, nr, kKeySide);
         }
-        commit(y0, nr);
+        float d[F::NL];
+        deltas(d, nr);
+        commit(y0, nr, d);
     };
     constexpr std::integral_constant<int, F::BR> kStep{};
     constexpr std::integral_constant<int, G::HR - F::BR> kRest{};
@@ -575,8 +589,12 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         }
 
         if (!more) break;
+        // dO . O of the next step's rows before the barrier: the query side, which stages most
+        // of them, would wait there for the key side anyway
+        float dnext[F::NL];
+        deltas(dnext, kStep);
         __syncthreads();  // every wave is done with this tile's LDS
-        commit(ny0, kStep);
+        commit(ny0, kStep, dnext);
         if (!below) stage_now(ny0 + F::BR, nbc, kRest);
         __syncthreads();
         cur = nxt;
