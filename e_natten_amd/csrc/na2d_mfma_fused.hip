@@ -77,16 +77,17 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
 
     const Shape &s = a.s;
     // Contiguous runs of column-major tiles per workgroup like make_runs, but of equal
-    // cost rather than equal length: a tile beside the border costs about 1.5 inner
-    // tiles here (measured), and whole columns of them (the first and last column of
-    // every image) would otherwise make their workgroups the last to finish.
+    // cost rather than equal length: a tile beside the border costs about 8/7 of an inner
+    // tile here (measured: the weights 3:2, 5:4, 8:7, 11:10 and 1:1 give 136.9, 132.6, 130.7,
+    // 131.9 and 134.6 us at B4 N4 128x128), and whole columns of them (the first and last
+    // column of every image) would otherwise make their workgroups the last to finish.
     Sched sc;
     {
         const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
         const int per = (ntiles + 7) >> 3;
         const int lo = xcd * per, hi = min(ntiles, lo + per);
         const int per_img = ts.tiles_r * ts.tiles_c;
-        // cost of tiles [0, t) in column-major order: 2 per inner tile, 3 per border tile
+        // cost of tiles [0, t) in column-major order: 7 per inner tile, 8 per border tile
         auto cost_to = [&](int t) __attribute__((always_inline)) {
             const int img = t / per_img, e = t % per_img;
             const int col = e / ts.tiles_r, row = e % ts.tiles_r;
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
             const int full_inner_cols = max(0, min(col, ts.ic0 + ts.ni_c) - ts.ic0);
             const long long inner = (long long)img * ts.ni_r * ts.ni_c +
                                     (long long)full_inner_cols * ts.ni_r + inner_in_col(col, row);
-            return 3ll * t - inner;
+            return 8ll * t - inner;
         };
         const long long c_lo = cost_to(lo), c_hi = cost_to(max(hi, lo));
         auto start_of = [&](int k) __attribute__((always_inline)) {
@@ -405,19 +406,19 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         } else {
             auto issue = [&](int part) __attribute__((always_inline)) { issue_as(part, kKeySide); };
             // ---- key side: this lane's key is column n of every product
-            if (inner) {
-                // Every window is centred: the queries are the (4+k-1)^2 pixels around
-                // the wave's keys and the mask depends on the lane only.  P and dS of all
-                // of them first, then dV and dK one after the other: one accumulator at a
-                // time leaves the registers to the next tile's rows.
-                const int ocol = (w & 1) * 4;
-                set_slots((w >> 1) * 4);
-                const int kyl = n >> 2, kxl = n & 3;
+            // The unrolled key-side body, for at most 64 queries (4 row tiles of 16): P and dS
+            // of all of them first, then dV and dK one after the other (one accumulator at a
+            // time leaves the registers to the next tile's rows).  The caller says where the
+            // queries are: arow(mt) is the LDS row of query mt*16 + n; stat(mt, i) and ok(mt, i)
+            // are the statistics of query mt*16 + g*4 + i and whether it attends this lane's
+            // key; trow(ks, h) is the LDS row of query ks*32 + h*16 + g*4 + n/4.
+            auto key_body = [&](int krow_lds, int64_t tok, auto arow, auto stat, auto ok_fn, auto trow)
+                                __attribute__((always_inline)) {
                 s16x8 pb[G::KSTEPS], dsb[G::KSTEPS];
                 {
                     s16x8 kreg[G::DS], vreg[G::DS];
                     {
-                        const typename G::ARow kp = G::a_row(lds_k, prow, g), vp = G::a_row(lds_v, prow, g);
+                        const typename G::ARow kp = G::a_row(lds_k, krow_lds, g), vp = G::a_row(lds_v, krow_lds, g);
 #pragma unroll
                         for (int ds = 0; ds < G::DS; ds++) {
                             kreg[ds] = *reinterpret_cast<const s16x8 *>(G::a_at(kp, ds));
@@ -428,29 +429,23 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                     for (int mt = 0; mt < G::MT; mt++) {
                         if (mt < 4) issue(mt);
                         f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
-                        const int row = tok_row(2 * mt, n >> 3, ocol + (n & 7));
+                        const int row = arow(mt);
                         const typename G::ARow qp = G::a_row(lds_q, row, g), gp = G::a_row(lds_g, row, g);
 #pragma unroll
                         for (int ds = 0; ds < G::DS; ds++) {
                             cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(qp, ds)), kreg[ds], cs);
                             cp = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(gp, ds)), vreg[ds], cp);
                         }
-                        // queries of accumulator rows g*4 .. g*4+3: halo row 2*mt + g/2,
-                        // columns 4*(g%2) .. +3, i.e. four consecutive LDS rows
-                        const float2 *stp = lds_stat + tok_row(2 * mt, g >> 1, ocol + 4 * (g & 1));
 #pragma unroll
                         for (int i = 0; i < 4; i++) {
-                            const float2 st = stp[i];
-                            const bool ok = ((unsigned)(2 * mt + (g >> 1) - kyl) < (unsigned)KS) &
-                                            ((unsigned)(4 * (g & 1) + i - kxl) < (unsigned)KS);
-                            const float p = __builtin_amdgcn_exp2f(keep_or_ninf(cs[i] * sc2 - st.x, ok));
+                            const float2 st = stat(mt, i);
+                            const float p = __builtin_amdgcn_exp2f(keep_or_ninf(cs[i] * sc2 - st.x, ok_fn(mt, i)));
                             pb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p);
                             dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
                         }
                     }
                 }
                 issue(4);
-                const int64_t tok = out_token();
                 auto second = [&](const short *lds_x, const s16x8 (&b)[G::KSTEPS], void *out, float mul)
                                   __attribute__((always_inline)) {
                     f32x4 acc[G::DT];
@@ -460,8 +455,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                     for (int ks = 0; ks < G::KSTEPS; ks++) {
                         typename G::TRow xt[2];
 #pragma unroll
-                        for (int h = 0; h < 2; h++)
-                            xt[h] = G::t_row(lds_x, tok_row(4 * ks + 2 * h, g >> 1, ocol + 4 * (g & 1) + (n >> 2)), n);
+                        for (int h = 0; h < 2; h++) xt[h] = G::t_row(lds_x, trow(ks, h), n);
 #pragma unroll
                         for (int mt = 0; mt < G::DT; mt++)
                             acc[mt] = mfma16<BF>(
@@ -472,58 +466,115 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 };
                 second(lds_g, pb, a.dv, 1.f);
                 second(lds_q, dsb, a.dk, s.scale);
-            } else {
-                // ---- key side of a tile beside the border.  The clamped windows make the
-                // set of queries that attend to the wave's 4x4 keys wider, up to SW + k/2
-                // per axis, and the relation depends on where a query's window starts:
-                // walk that region 32 queries at a time, with one bit per region row /
-                // column telling whether that query row / column attends this lane's key
-                // row / column.  The loop is rolled
-                // (unrolled, the addresses of the whole region would be formed up front).
-                const int ky0 = cur.r0 + (w >> 1) * 4, kx0 = cur.c0 + (w & 1) * 4;
-                // query rows / columns that attend the wave's key rows / columns: SW of them
-                // away from the border, SW - k/2 or SW + k/2 beside it
-                const int qr0 = inv_lo(ky0, KS), qc0 = inv_lo(kx0, KS);
-                const int nr = inv_hi(ky0 + 3, s.H, KS) - qr0, nc = inv_hi(kx0 + 3, s.W, KS) - qc0;
+            };
+            const bool edge_r = tr == 0 || tr == ts.tiles_r - 1, edge_c = tc == 0 || tc == ts.tiles_c - 1;
+            if (inner) {
+                // Every window is centred: the queries are the (4+k-1)^2 pixels around the
+                // wave's 4x4 keys, 8 to a row, and the mask depends on the lane only.
+                const int ocol = (w & 1) * 4;
+                set_slots((w >> 1) * 4);
+                const int kyl = n >> 2, kxl = n & 3;
+                key_body(
+                    prow, out_token(),
+                    [&](int mt) __attribute__((always_inline)) { return tok_row(2 * mt, n >> 3, ocol + (n & 7)); },
+                    // queries of accumulator rows g*4 .. g*4+3: halo row 2*mt + g/2, columns
+                    // 4*(g%2) .. +3, i.e. four consecutive LDS rows
+                    [&](int mt, int i) __attribute__((always_inline)) {
+                        return lds_stat[tok_row(2 * mt, g >> 1, ocol + 4 * (g & 1)) + i];
+                    },
+                    [&](int mt, int i) __attribute__((always_inline)) {
+                        return ((unsigned)(2 * mt + (g >> 1) - kyl) < (unsigned)KS) &
+                               ((unsigned)(4 * (g & 1) + i - kxl) < (unsigned)KS);
+                    },
+                    [&](int ks, int h) __attribute__((always_inline)) {
+                        return tok_row(4 * ks + 2 * h, g >> 1, ocol + 4 * (g & 1) + (n >> 2));
+                    });
+            } else if (edge_r != edge_c) {
+                // ---- key side of a tile beside one border.  The clamped windows put more
+                // queries on the keys 3 and 4 pixels from a border and fewer on those beside
+                // it, so with 4x4 blocks of keys the two waves away from the border would have
+                // 10 rows of queries and the other two 6.  The waves therefore take strips of
+                // keys that run away from the border, 8 x 2 beside the top or bottom and 2 x 8
+                // beside the left or right: every wave then has the 10 x 6 queries of its strip,
+                // 60 of the 64 that the unrolled body serves, numbered row-major.
+                const bool tall = edge_r;
+                const int kr0 = tall ? 0 : 2 * w, kc0 = tall ? 2 * w : 0;  // strip origin in the tile
+                const int krn = tall ? 8 : 2, kcn = tall ? 2 : 8;
+                const int ky = cur.r0 + kr0 + (tall ? n >> 1 : n >> 3);   // this lane's key
+                const int kx = cur.c0 + kc0 + (tall ? n & 1 : n & 7);
+                // query rows / columns that attend the strip's key rows / columns
+                const int qr0 = inv_lo(cur.r0 + kr0, KS), qc0 = inv_lo(cur.c0 + kc0, KS);
+                const int nr = inv_hi(cur.r0 + kr0 + krn - 1, s.H, KS) - qr0;
+                const int nc = inv_hi(cur.c0 + kc0 + kcn - 1, s.W, KS) - qc0;
                 const int orow = qr0 - br, ocol = qc0 - bc;
-                // The region is numbered along its shorter side where that has at most SW
-                // queries (8 per line, else 16), so that its lines fill the 32-query steps:
-                // 2 or 3 steps for a wave beside one border, 5 only in a corner.
-                const bool tr = nc > G::SW && nr <= G::SW;  // lines are columns
-                const int nmaj = tr ? nc : nr, nmin = tr ? nr : nc;
-                const int lsh = nmin > G::SW ? 4 : 3;
-                const int nks = ((nmaj << lsh) + 31) >> 5;
+                const int nq = nr * nc;                   // <= 64 (FGeo::FITS)
+                const int magic = (65536 + nc - 1) / nc;  // tk * magic >> 16 == tk / nc for tk < 2048
                 unsigned rmask = 0, cmask = 0;
 #pragma unroll
                 for (int r = 0; r < F::SWB; r++) {
                     const int qy = qr0 + r, qx = qc0 + r;
-                    const bool oky = (r < nr) & ((unsigned)(py - win_start(qy, s.H, KS)) < (unsigned)KS);
-                    const bool okx = (r < nc) & ((unsigned)(px - win_start(qx, s.W, KS)) < (unsigned)KS);
+                    const bool oky = (r < nr) & ((unsigned)(ky - win_start(qy, s.H, KS)) < (unsigned)KS);
+                    const bool okx = (r < nc) & ((unsigned)(kx - win_start(qx, s.W, KS)) < (unsigned)KS);
                     rmask |= (oky ? 1u : 0u) << r;
                     cmask |= (okx ? 1u : 0u) << r;
                 }
-                // region (row, column) of query number tk; numbers beyond the region have
-                // a row or column whose mask bit is clear
-                auto reg_r = [&](int tk) __attribute__((always_inline)) {
-                    const int maj = tk >> lsh, mn = tk & ((1 << lsh) - 1);
-                    return tr ? mn : maj;
-                };
-                auto reg_c = [&](int tk) __attribute__((always_inline)) {
-                    const int maj = tk >> lsh, mn = tk & ((1 << lsh) - 1);
-                    return tr ? maj : mn;
-                };
                 auto row_of = [&](int tk) __attribute__((always_inline)) {
-                    const int r = reg_r(tk), c = reg_c(tk);
-                    return ((r < nr) & (c < nc)) ? block_row(orow + r, ocol + c) : (int)G::ZROW;
+                    const int r = (tk * magic) >> 16, c = tk - r * nc;
+                    return tk < nq ? block_row(orow + r, ocol + c) : (int)G::ZROW;
+                };
+                key_body(
+                    block_row(ky - br, kx - bc), (((int64_t)cur.bb * s.N + cur.nn) * s.H + ky) * s.W + kx,
+                    [&](int mt) __attribute__((always_inline)) { return row_of(mt * 16 + n); },
+                    [&](int mt, int i) __attribute__((always_inline)) { return lds_stat[row_of(mt * 16 + g * 4 + i)]; },
+                    [&](int mt, int i) __attribute__((always_inline)) {
+                        const int tk = mt * 16 + g * 4 + i, r = (tk * magic) >> 16, c = tk - r * nc;
+                        return (tk < nq) & (((rmask >> r) & (cmask >> c) & 1u) != 0u);
+                    },
+                    [&](int ks, int h) __attribute__((always_inline)) {
+                        return row_of(ks * 32 + h * 16 + g * 4 + (n >> 2));
+                    });
+            } else {
+                // ---- key side of a corner tile (and of every tile of an image with one tile
+                // row or column).  The clamped windows make the set of queries that attend to
+                // the wave's 4x4 keys wider, up to SW + k/2 per axis, more than the unrolled
+                // body serves, and the relation depends on where a query's window starts:
+                // walk that region 32 queries at a time, with one bit per region row /
+                // column telling whether that query row / column attends this lane's key
+                // row / column.  The loop is rolled
+                // (unrolled, the addresses of the whole region would be formed up front).
+                const int kr0 = (w >> 1) * 4, kc0 = (w & 1) * 4, krn = 4, kcn = 4;
+                const int ky = py, kx = px;
+                const int krow_lds = prow;
+                // query rows / columns that attend the block's key rows / columns
+                const int qr0 = inv_lo(cur.r0 + kr0, KS), qc0 = inv_lo(cur.c0 + kc0, KS);
+                const int nr = inv_hi(cur.r0 + kr0 + krn - 1, s.H, KS) - qr0;
+                const int nc = inv_hi(cur.c0 + kc0 + kcn - 1, s.W, KS) - qc0;
+                const int orow = qr0 - br, ocol = qc0 - bc;
+                // the region's queries are numbered row-major, nc to a row
+                const int nq = nr * nc, nks = (nq + 31) >> 5;
+                const int magic = (65536 + nc - 1) / nc;  // tk * magic >> 16 == tk / nc for tk < 2048
+                unsigned rmask = 0, cmask = 0;
+#pragma unroll
+                for (int r = 0; r < F::SWB; r++) {
+                    const int qy = qr0 + r, qx = qc0 + r;
+                    const bool oky = (r < nr) & ((unsigned)(ky - win_start(qy, s.H, KS)) < (unsigned)KS);
+                    const bool okx = (r < nc) & ((unsigned)(kx - win_start(qx, s.W, KS)) < (unsigned)KS);
+                    rmask |= (oky ? 1u : 0u) << r;
+                    cmask |= (okx ? 1u : 0u) << r;
+                }
+                auto row_of = [&](int tk) __attribute__((always_inline)) {
+                    const int r = (tk * magic) >> 16, c = tk - r * nc;
+                    return tk < nq ? block_row(orow + r, ocol + c) : (int)G::ZROW;
                 };
                 auto ok_of = [&](int tk) __attribute__((always_inline)) {
-                    return ((rmask >> reg_r(tk)) & (cmask >> reg_c(tk)) & 1u) != 0u;
+                    const int r = (tk * magic) >> 16, c = tk - r * nc;
+                    return (tk < nq) & (((rmask >> r) & (cmask >> c) & 1u) != 0u);
                 };
                 // this lane's key and value rows are read from LDS where they are used
                 // (the registers do not hold them beside the two accumulators and the
                 // next tile's rows)
-                const int pkey = G::key(prow), kvh = pkey >> 2;
-                int kvoff = prow * G::PITCH + ((g ^ (pkey & 3)) << 3);
+                const int pkey = G::key(krow_lds), kvh = pkey >> 2;
+                int kvoff = krow_lds * G::PITCH + ((g ^ (pkey & 3)) << 3);
                 f32x4 dk[G::DT], dv[G::DT];
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++) {
@@ -582,7 +633,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 issue(2);
                 issue(3);
                 issue(4);
-                const int64_t tok = out_token();
+                const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + ky) * s.W + kx;
                 store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
                 store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
             }
