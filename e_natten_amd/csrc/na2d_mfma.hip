@@ -1105,11 +1105,15 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
 
         // The fused backward where it is built and measured faster than the two passes:
         // enough tiles for every CU to walk a while, images large enough that the tiles
-        // beside the border (dearer than an inner tile there) are few, and at most
-        // 48 tiles per workgroup: its workgroups take their tiles in one contiguous run,
-        // so with several columns each they stop meeting their neighbours in L2, while
-        // the two-pass kernels deal columns out in turn (plan_runs) and keep doing so.
-        const bool fused_pays = nb >= 1024 && nb <= 12288 && tiles_r >= 12 && tiles_c >= 12;
+        // beside the border (dearer than an inner tile there) are few, and either at most
+        // 48 tiles per workgroup or whole columns that come out even when dealt in rounds
+        // (the rule of bwd_fused_mfma's schedule): with several columns in one contiguous
+        // run the workgroups stop meeting their neighbours in L2, while the two-pass
+        // kernels deal columns out in turn (plan_runs) and keep doing so.
+        const int64_t per_xcd = (nb + 7) / 8, xcd_cols = per_xcd / tiles_r;
+        const bool dealt = nb % 8 == 0 && per_xcd % tiles_r == 0 && xcd_cols >= 64 &&
+                           ((xcd_cols + 31) / 32 * 32 - xcd_cols) * 16 <= xcd_cols;
+        const bool fused_pays = nb >= 1024 && (nb <= 12288 || dealt) && tiles_r >= 12 && tiles_c >= 12;
         if (path != ENATTEN_PATH_MFMA_SPLIT && fused_bwd_supported(a) &&
             (path == ENATTEN_PATH_MFMA_FUSED || fused_pays)) {
             const int rc = launch_bwd_fused(a, BF, ts, nb, st);

@@ -82,6 +82,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     // 131.9 and 134.6 us at B4 N4 128x128), and whole columns of them (the first and last
     // column of every image) would otherwise make their workgroups the last to finish.
     Sched sc;
+    int deal_ncols = 0, deal_lo = 0, seg_end = 0, deal_round = 0;  // columns dealt in rounds, see below
     {
         const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
         const int per = (ntiles + 7) >> 3;
@@ -115,8 +116,40 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         sc.t = start_of(slot);
         sc.t_end = slot + 1 == slots ? max(hi, lo) : start_of(slot + 1);
         sc.step = 1;
+        // Where an XCD has two or more whole columns per workgroup, a contiguous run would
+        // put its workgroups on columns that are never adjacent at the same time, and the
+        // block columns that neighbouring tiles share would all come from HBM.  The XCD's
+        // columns are then dealt in rounds instead: in round r workgroup `slot` walks column
+        // r * slots + (slot + 2r) % slots, so that at any time the workgroups are on
+        // neighbouring columns at the same height, and the rotation by 2r spreads the dearer
+        // first and last columns of the images over the workgroups (B8 N8 128x128: 617 ->
+        // 475 us; B4 N4 256x256: 599 -> 511).  Only where the rounds come out even: a last
+        // round that leaves many workgroups without a column costs more than the sharing
+        // gains (B4 N10 128x128, 2.5 rounds: 344 -> 371 us), and so do columns cut into parts
+        // to make rounds (B2 N4 160x160: 113 -> 122 us).
+        if (per % ts.tiles_r == 0 && hi - lo == per) {
+            const int ncols = per / ts.tiles_r, rounds = (ncols + slots - 1) / slots;
+            if (ncols >= 2 * slots && (rounds * slots - ncols) * 16 <= ncols) {
+                deal_ncols = ncols;
+                deal_lo = lo;
+                sc.t = lo + slot * ts.tiles_r;  // round 0: column `slot`
+                seg_end = sc.t + ts.tiles_r;
+                sc.t_end = hi;
+            }
+        }
     }
     if (sc.t >= sc.t_end) return;
+    // the tile after t in this workgroup's walk, or sc.t_end
+    auto tile_after = [&](int t, int &round) __attribute__((always_inline)) {
+        if (deal_ncols == 0 || t + 1 < seg_end) return t + 1;
+        const int slots = gridDim.x >> 3, slot = blockIdx.x >> 3;
+        round++;
+        const int col = round * slots + (slot + 2 * round) % slots;
+        if (col >= deal_ncols) return sc.t_end;
+        const int t0 = deal_lo + col * ts.tiles_r;
+        seg_end = t0 + ts.tiles_r;
+        return t0;
+    };
     const int tid = threadIdx.x;
     if (tid < G::CPR) {
         const u32x4 z = {0u, 0u, 0u, 0u};
@@ -295,7 +328,8 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
             for (int i = 0; i < F::NL; i++) asm volatile("" : "=v"(fresh.v[i]));
             qst = fresh; gst = fresh; kst = fresh; vst = fresh; ost = fresh;
         }
-        const int tn = sc.t + 1;
+        int round_n = deal_round;
+        const int tn = tile_after(sc.t, round_n);
         const bool more = tn < sc.t_end;
         const Tile nxt = more ? tile_of_cm(tn, ts.tiles_r, ts.tiles_c, s.N) : cur;
         // the tile below in the same image: its block shares k-1 rows with this one
@@ -650,6 +684,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         __syncthreads();
         cur = nxt;
         sc.t = tn;
+        deal_round = round_n;
     }
 }
 
