@@ -1103,17 +1103,12 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         const int64_t slabs = (int64_t)a.s.B * a.s.N;
         const int64_t n_inner = slabs * ts.ni_r * ts.ni_c, n_frame = nb - n_inner;
 
-        // The fused backward where it is built and measured faster than the two passes:
-        // enough tiles for every CU to walk a while, images large enough that the tiles
-        // beside the border (dearer than an inner tile there) are few, and either at most
-        // 48 tiles per workgroup or whole columns that come out even when dealt in rounds
-        // (the rule of bwd_fused_mfma's schedule): with several columns in one contiguous
-        // run the workgroups stop meeting their neighbours in L2, while the two-pass
-        // kernels deal columns out in turn (plan_runs) and keep doing so.
-        const int64_t per_xcd = (nb + 7) / 8, xcd_cols = per_xcd / tiles_r;
-        const bool dealt = nb % 8 == 0 && per_xcd % tiles_r == 0 && xcd_cols >= 64 &&
-                           ((xcd_cols + 31) / 32 * 32 - xcd_cols) * 16 <= xcd_cols;
-        const bool fused_pays = nb >= 1024 && (nb <= 12288 || dealt) && tiles_r >= 12 && tiles_c >= 12;
+        // The fused backward where it is built (fused_bwd_supported), except for images of
+        // fewer than 4 tiles a side, where most tiles are corner tiles and the two passes
+        // were measured 4-10% faster (B16 N8 16x16: 26.3 against 29.1 us; B32 N8 24x24: 93
+        // against 98).  Elsewhere it is 5-25% faster than the two passes, from B4 N4 32x32
+        // (17.7 against 24.1 us) to B16 N8 128x128 (938 against 1174).
+        const bool fused_pays = tiles_r >= 4 && tiles_c >= 4;
         if (path != ENATTEN_PATH_MFMA_SPLIT && fused_bwd_supported(a) &&
             (path == ENATTEN_PATH_MFMA_FUSED || fused_pays)) {
             const int rc = launch_bwd_fused(a, BF, ts, nb, st);

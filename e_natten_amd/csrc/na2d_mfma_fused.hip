@@ -47,8 +47,8 @@ struct FGeo {
     // Key side beside the border: the queries that attend to a wave's 4x4 keys
     // span up to SW + k/2 rows and columns there.
     static constexpr int SWB = G::SW + KS / 2;
-    static constexpr size_t LDS_BYTES =
-        (size_t)4 * G::ROWS * G::PITCH * sizeof(short) + (size_t)G::ROWS * sizeof(float2);
+    static constexpr size_t LDS_BYTES = (size_t)4 * G::ROWS * G::PITCH * sizeof(short) +
+                                        (size_t)G::ROWS * sizeof(float2) + 4 * 64 * sizeof(int);
     static constexpr bool FITS = LDS_BYTES <= 160 * 1024 && G::HR - BR <= BR && SWB <= 16 &&
                                  SWB <= G::HR;
 };
@@ -74,47 +74,25 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
     __shared__ float2 lds_stat[G::ROWS];  // (log-sum-exp * log2(e), dO . O) per staged query
+    // per key-side wave, for a tile beside a border: LDS row | region row << 16 | region
+    // column << 20 of each of its 64 query numbers
+    __shared__ int lds_qtab[4 * 64];
 
     const Shape &s = a.s;
-    // Contiguous runs of column-major tiles per workgroup like make_runs, but of equal
-    // cost rather than equal length: a tile beside the border costs about 8/7 of an inner
-    // tile here (measured: the weights 3:2, 5:4, 8:7, 11:10 and 1:1 give 136.9, 132.6, 130.7,
-    // 131.9 and 134.6 us at B4 N4 128x128), and whole columns of them (the first and last
-    // column of every image) would otherwise make their workgroups the last to finish.
+    // One contiguous run of column-major tiles per workgroup, all of the same length: a tile
+    // beside a border costs about as much as an inner one since its key side runs the
+    // unrolled body too (with run weights border : inner of 8:7, 16:15, 32:31 and 1:1 the
+    // kernel takes 130.5, 128.6, 128.8 and 127.5 us at B4 N4 128x128), and runs of equal
+    // length keep the workgroups of an XCD on neighbouring columns at the same height
+    // where a run is one column.
     Sched sc;
     int deal_ncols = 0, deal_lo = 0, seg_end = 0, deal_round = 0;  // columns dealt in rounds, see below
     {
         const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
         const int per = (ntiles + 7) >> 3;
-        const int lo = xcd * per, hi = min(ntiles, lo + per);
-        const int per_img = ts.tiles_r * ts.tiles_c;
-        // cost of tiles [0, t) in column-major order: 7 per inner tile, 8 per border tile
-        auto cost_to = [&](int t) __attribute__((always_inline)) {
-            const int img = t / per_img, e = t % per_img;
-            const int col = e / ts.tiles_r, row = e % ts.tiles_r;
-            auto inner_in_col = [&](int c, int rows) __attribute__((always_inline)) {
-                const bool cin = c >= ts.ic0 && c < ts.ic0 + ts.ni_c;
-                return cin ? max(0, min(rows, ts.ir0 + ts.ni_r) - ts.ir0) : 0;
-            };
-            const int full_inner_cols = max(0, min(col, ts.ic0 + ts.ni_c) - ts.ic0);
-            const long long inner = (long long)img * ts.ni_r * ts.ni_c +
-                                    (long long)full_inner_cols * ts.ni_r + inner_in_col(col, row);
-            return 8ll * t - inner;
-        };
-        const long long c_lo = cost_to(lo), c_hi = cost_to(max(hi, lo));
-        auto start_of = [&](int k) __attribute__((always_inline)) {
-            // first tile t in [lo, hi] with cost_to(t) - c_lo >= k * (c_hi - c_lo) / slots
-            const long long want = c_lo + (c_hi - c_lo) * k / slots;
-            int a0 = lo, a1 = max(hi, lo);
-            while (a0 < a1) {
-                const int mid = (a0 + a1) >> 1;
-                if (cost_to(mid) >= want) a1 = mid;
-                else a0 = mid + 1;
-            }
-            return a0;
-        };
-        sc.t = start_of(slot);
-        sc.t_end = slot + 1 == slots ? max(hi, lo) : start_of(slot + 1);
+        const int lo = xcd * per, hi = max(min(ntiles, lo + per), lo);
+        sc.t = lo + (int)((long long)(hi - lo) * slot / slots);
+        sc.t_end = lo + (int)((long long)(hi - lo) * (slot + 1) / slots);
         sc.step = 1;
         // Where an XCD has two or more whole columns per workgroup, a contiguous run would
         // put its workgroups on columns that are never adjacent at the same time, and the
@@ -123,19 +101,15 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         // r * slots + (slot + 2r) % slots, so that at any time the workgroups are on
         // neighbouring columns at the same height, and the rotation by 2r spreads the dearer
         // first and last columns of the images over the workgroups (B8 N8 128x128: 617 ->
-        // 475 us; B4 N4 256x256: 599 -> 511).  Only where the rounds come out even: a last
-        // round that leaves many workgroups without a column costs more than the sharing
-        // gains (B4 N10 128x128, 2.5 rounds: 344 -> 371 us), and so do columns cut into parts
-        // to make rounds (B2 N4 160x160: 113 -> 122 us).
-        if (per % ts.tiles_r == 0 && hi - lo == per) {
-            const int ncols = per / ts.tiles_r, rounds = (ncols + slots - 1) / slots;
-            if (ncols >= 2 * slots && (rounds * slots - ncols) * 16 <= ncols) {
-                deal_ncols = ncols;
-                deal_lo = lo;
-                sc.t = lo + slot * ts.tiles_r;  // round 0: column `slot`
-                seg_end = sc.t + ts.tiles_r;
-                sc.t_end = hi;
-            }
+        // 475 us; B4 N4 256x256: 599 -> 511).  The columns that do not fill a round are
+        // shared out as one more contiguous run per workgroup.  (Columns cut into parts to
+        // make rounds where there are fewer were measured slower, B2 N4 160x160: 113 -> 122 us.)
+        if (per % ts.tiles_r == 0 && hi - lo == per && per / ts.tiles_r >= 2 * slots) {
+            deal_ncols = per / ts.tiles_r;
+            deal_lo = lo;
+            sc.t = lo + slot * ts.tiles_r;  // round 0: column `slot`
+            seg_end = sc.t + ts.tiles_r;
+            sc.t_end = hi;
         }
     }
     if (sc.t >= sc.t_end) return;
@@ -144,11 +118,19 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         if (deal_ncols == 0 || t + 1 < seg_end) return t + 1;
         const int slots = gridDim.x >> 3, slot = blockIdx.x >> 3;
         round++;
-        const int col = round * slots + (slot + 2 * round) % slots;
-        if (col >= deal_ncols) return sc.t_end;
-        const int t0 = deal_lo + col * ts.tiles_r;
-        seg_end = t0 + ts.tiles_r;
-        return t0;
+        const int full = deal_ncols / slots;  // rounds in which every workgroup has a column
+        if (round < full) {
+            const int t0 = deal_lo + (round * slots + (slot + 2 * round) % slots) * ts.tiles_r;
+            seg_end = t0 + ts.tiles_r;
+            return t0;
+        }
+        if (round == full) {
+            const int rest_lo = deal_lo + full * slots * ts.tiles_r, rest = sc.t_end - rest_lo;
+            const int t0 = rest_lo + (int)((long long)rest * slot / slots);
+            seg_end = rest_lo + (int)((long long)rest * (slot + 1) / slots);
+            if (t0 < seg_end) return t0;
+        }
+        return sc.t_end;
     };
     const int tid = threadIdx.x;
     if (tid < G::CPR) {
@@ -552,20 +534,27 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                     rmask |= (oky ? 1u : 0u) << r;
                     cmask |= (okx ? 1u : 0u) << r;
                 }
-                auto row_of = [&](int tk) __attribute__((always_inline)) {
-                    const int r = (tk * magic) >> 16, c = tk - r * nc;
-                    return tk < nq ? block_row(orow + r, ocol + c) : (int)G::ZROW;
+                // Every lane works out where one query number lives; the wave reads the table
+                // back wherever the body asks for a query (24 times per lane).  Numbers past
+                // the region get the zero row and a row bit that no key has.
+                int *qtab = lds_qtab + w * 64;
+                {
+                    const int r = (l * magic) >> 16, c = l - r * nc;
+                    qtab[l] = l < nq ? block_row(orow + r, ocol + c) | (r << 16) | (c << 20)
+                                     : (int)G::ZROW | (15 << 16);
+                }
+                auto ok_at = [&](int e) __attribute__((always_inline)) {
+                    return ((rmask >> ((e >> 16) & 15)) & (cmask >> (e >> 20)) & 1u) != 0u;
                 };
                 key_body(
                     block_row(ky - br, kx - bc), (((int64_t)cur.bb * s.N + cur.nn) * s.H + ky) * s.W + kx,
-                    [&](int mt) __attribute__((always_inline)) { return row_of(mt * 16 + n); },
-                    [&](int mt, int i) __attribute__((always_inline)) { return lds_stat[row_of(mt * 16 + g * 4 + i)]; },
+                    [&](int mt) __attribute__((always_inline)) { return qtab[mt * 16 + n] & 0xffff; },
                     [&](int mt, int i) __attribute__((always_inline)) {
-                        const int tk = mt * 16 + g * 4 + i, r = (tk * magic) >> 16, c = tk - r * nc;
-                        return (tk < nq) & (((rmask >> r) & (cmask >> c) & 1u) != 0u);
+                        return lds_stat[qtab[mt * 16 + g * 4 + i] & 0xffff];
                     },
+                    [&](int mt, int i) __attribute__((always_inline)) { return ok_at(qtab[mt * 16 + g * 4 + i]); },
                     [&](int ks, int h) __attribute__((always_inline)) {
-                        return row_of(ks * 32 + h * 16 + g * 4 + (n >> 2));
+                        return qtab[ks * 32 + h * 16 + g * 4 + (n >> 2)] & 0xffff;
                     });
             } else {
                 // ---- key side of a corner tile (and of every tile of an image with one tile
