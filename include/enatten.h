@@ -59,10 +59,10 @@ int enatten2d_kernel_path(int D, int kernel_size, int dtype);
  * Steer dispatch: 0 = automatic (default), ENATTEN_PATH_SIMT = never use the
  * matrix-core kernels.  The matrix-core backward has two forms: two passes (dQ, then
  * dK/dV) and one fused kernel that stages q, k, v, dO once (built for head_dim 128,
- * kernel_size 5, image sides that are multiples of 8, contiguous rows).  Automatic
- * dispatch takes the fused form where it is built and measured faster (2048 to 12288
- * tiles of 8x8 pixels in the call and at least 12 tiles along each image side);
- * ENATTEN_PATH_MFMA_FUSED takes it wherever it is built, ENATTEN_PATH_MFMA_SPLIT never.
+ * kernel_size 5, image sides that are multiples of 8; the 1D operator has one for
+ * kernel_size <= 17, and for head_dim <= 64 beyond).  Automatic dispatch and
+ * ENATTEN_PATH_MFMA_FUSED take the fused form wherever it is built (it was measured
+ * faster at every size), ENATTEN_PATH_MFMA_SPLIT never.
  * Process-wide; meant for tests and tuning.  Returns the previous setting.
  */
 int enatten_set_path(int path);
