@@ -69,11 +69,15 @@ def test_config2_bf16_readme_shape(side, path):
 @pytest.mark.parametrize("shape,dtype", [((1, 1, 8, 8, 128), BF), ((1, 2, 16, 24, 128), BF),
                                          ((4, 4, 32, 32, 128), BF), ((2, 3, 64, 40, 128), BF),
                                          ((4, 4, 128, 128, 128), BF), ((1, 3, 40, 72, 128), F16),
+                                         ((2, 2, 8, 48, 128), BF), ((3, 1, 56, 8, 128), F16),
+                                         ((2, 1, 16, 16, 128), BF), ((1, 2, 24, 24, 128), BF),
+                                         ((20, 16, 16, 16, 128), BF),  # 80 columns per XCD: dealt in two rounds and a remainder
                                          ((1, 2, 37, 50, 128), BF)])
 def test_fused_backward_path(shape, dtype, _lib):
     # the fused backward (dQ, dK, dV of every tile from one staging of q, k, v, dO),
-    # forced wherever it is built, against the oracle: images that are all border, mixed, fp16; the last shape
-    # has sides that are no multiples of 8 and is served by the two-pass kernels
+    # forced wherever it is built, against the oracle: images that are all border (one, two and three tiles a
+    # side: corner and edge tiles only), mixed, fp16, columns dealt in rounds; the last shape has sides that
+    # are no multiples of 8 and is served by the two-pass kernels
     from e_natten_amd._lib import PATH_MFMA_FUSED
     prev = _lib.enatten_set_path(PATH_MFMA_FUSED)
     try:
