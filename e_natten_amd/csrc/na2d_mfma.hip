@@ -176,6 +176,122 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
     }
 }
 
+// ------------------------------------------------------------------ forward, one halo in LDS at a time
+// The forward for halos of which LDS holds two only once per CU (head_dim 128 with
+// kernel_size 7 and 9), like bwd_dq2_mfma: K rows first (logits, softmax; P stays in
+// registers as 16-bit values) while the tile's V rows are in flight, V over K behind a
+// barrier, then O^T = V^T P^T while the next tile's K rows are in flight.  Two workgroups
+// per CU, four barriers per tile; 8x8 tiles, no column walk.
+template <bool BF, int D, int KS>
+__global__ __launch_bounds__(256, 2) void fwd2_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles) {
+    using G = Geo<D, KS>;
+    __shared__ __attribute__((aligned(16))) short lds_x[G::ROWS * G::PITCH];
+    const Shape &s = a.s;
+    Sched sc = make_sched(ntiles, blockIdx.x, gridDim.x);
+    if (sc.t >= sc.t_end) return;
+    zero_row<D, KS>(lds_x);
+
+    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const float sc2 = s.scale * kLog2e;
+    const HaloPlan<D, KS> plan = make_plan<D, KS>();
+    HaloRegs<D, KS> st;
+    s16x8 qnext[G::DS];
+    auto fetch_rows = [&](const View &vw, const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
+        halo_fetch<D, KS>(st, plan, image<short>(vw, tl), vw.sh, vw.sw, lq.hr0, lq.hc0, s.H, s.W);
+    };
+    auto fetch_q = [&](const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
+        const short *qp = image<short>(a.q, tl) + lq.qr * a.q.sh + lq.qc * a.q.sw + g * 8;
+#pragma unroll
+        for (int ds = 0; ds < G::DS; ds++) qnext[ds] = *reinterpret_cast<const s16x8 *>(qp + ds * 32);
+    };
+    Tile cur = tile_of(sc.t, tiles_r, tiles_c, s.N);
+    LaneQ lq = lane_query<KS>(cur, s, wave, n);
+    fetch_rows(a.k, cur, lq);
+    fetch_q(cur, lq);
+    for (;;) {
+        halo_commit<D, KS>(lds_x, plan, st);  // K
+        s16x8 qreg[G::DS];
+#pragma unroll
+        for (int ds = 0; ds < G::DS; ds++) qreg[ds] = qnext[ds];
+        __syncthreads();
+        fetch_rows(a.v, cur, lq);
+        auto trow = [&](int tk) __attribute__((always_inline)) { return G::token_row(tk, lq.orow, lq.ocol); };
+        s16x8 pb[G::KSTEPS];
+        float mx = -INFINITY, sum = 0.f;
+        if (lq.wave_on) {
+            f32x4 acc[G::MT];
+#pragma unroll
+            for (int mt = 0; mt < G::MT; mt++) {
+                const typename G::ARow kp = G::a_row(lds_x, trow(mt * 16 + n), g);
+                f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ds = 0; ds < G::DS; ds++)
+                    c = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(kp, ds)), qreg[ds], c);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int tk = mt * 16 + g * 4 + i;
+                    const int kr = tk / G::SWC, kc = tk % G::SWC;
+                    const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
+                                    (unsigned)(kc - lq.dc) < (unsigned)KS;
+                    c[i] = ok ? c[i] * sc2 : -INFINITY;
+                    mx = fmaxf(mx, c[i]);
+                }
+                acc[mt] = c;
+            }
+            mx = col_max(mx);
+#pragma unroll
+            for (int mt = 0; mt < G::MT; mt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float p = __builtin_amdgcn_exp2f(acc[mt][i] - mx);
+                    sum += p;
+                    pb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p);
+                }
+            sum = col_sum(sum);
+        }
+        __syncthreads();                      // every wave has read K
+        halo_commit<D, KS>(lds_x, plan, st);  // V
+        __syncthreads();
+
+        const int tn = sched_peek(sc);
+        const bool more = tn < sc.t_end;
+        Tile nxt = cur;
+        LaneQ lqn = lq;
+        if (more) {
+            nxt = tile_of(tn, tiles_r, tiles_c, s.N);
+            lqn = lane_query<KS>(nxt, s, wave, n);
+            fetch_rows(a.k, nxt, lqn);
+            fetch_q(nxt, lqn);
+        }
+        if (lq.wave_on) {
+            f32x4 o[G::DT];
+#pragma unroll
+            for (int mt = 0; mt < G::DT; mt++) o[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < G::KSTEPS; ks++) {
+                typename G::TRow vp[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                    vp[h] = G::t_row(lds_x, trow(ks * 32 + h * 16 + g * 4 + (n >> 2)), n);
+#pragma unroll
+                for (int mt = 0; mt < G::DT; mt++)
+                    o[mt] = mfma16<BF>(
+                        cat(lds_read_tr(G::t_at(vp[0], mt)), lds_read_tr(G::t_at(vp[1], mt))), pb[ks],
+                        o[mt]);
+            }
+            store_token<BF, D>(const_cast<short *>(image<short>(a.o, cur)) + lq.qr * a.o.sh + lq.qc * a.o.sw,
+                               g, o, 1.f / sum, lq.live);
+            if (lq.live && a.lse && g == 0)
+                a.lse[lq.tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
+        }
+        if (!more) break;
+        __syncthreads();  // every wave has read V
+        cur = nxt;
+        lq = lqn;
+        sched_advance(sc, tn);
+    }
+}
+
 // ------------------------------------------------------------------ dQ
 // Query-centric like the forward: recompute P from the saved log-sum-exp, form
 // dP^T = V dO^T on the same halo, dS = P * (dP - delta) with delta = sum_j P_j dP_j
@@ -1048,6 +1164,16 @@ constexpr bool kDq2Built = D == 64 && Geo<D, KS>::WAVES == 1 && !kTallDqBuilt<D,
 // queries (Geo's SP): where the staged queries leave LDS for one workgroup per CU, a
 // SIMD then still holds two waves.  Built for head_dim 64 (the partial sums of the
 // second wave pass through 32 KB of LDS there).
+// The forward with one halo in LDS at a time (fwd2_mfma), for head_dim 128 where two halos
+// leave LDS for one workgroup per CU (kernel_size 7 and 9).  It pays from four tiles per
+// workgroup of its grid on (us, fwd_mfma -> fwd2_mfma, bf16, 128x128 images): k = 7
+// B2 N4 48.6 -> 44.2, B4 N4 91.8 -> 84.4, B8 N8 364 -> 353; k = 9 B2 N4 56.6 -> 54.2,
+// B4 N4 106.6 -> 103.0; with fewer tiles the walk down the columns of fwd_mfma, or its
+// single workgroup per CU, is as fast or faster (B1 N2: 14.8 -> 16.3).
+template <int D, int KS>
+constexpr bool kFwd2Built = D == 128 && Geo<D, KS>::WAVES == 1 &&
+                            2 * (Geo<D, KS>::ROWS * Geo<D, KS>::PITCH * 2 + 1024) <= 160 * 1024;
+
 template <int D, int KS>
 constexpr int kDkdvSplit = D == 64 && Geo<D, KS>::WAVES == 1 ? 2 : 1;
 
@@ -1066,6 +1192,15 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
                 ProfScope prof(ENATTEN_KERNEL_FWD, "fwd_mfma", st);
                 hipLaunchKernelGGL((fwd_mfma<BF, D, KS, false, 8>), dim3(grid), dim3(G8::NT), 0, st, a,
                                    tall_r, tiles_c, (int)nb8, Runs{0, 0});
+                return check_launch("enatten2d_fwd");
+            }
+        }
+        if constexpr (kFwd2Built<D, KS>) {
+            const int grid = persistent_grid<fwd2_mfma<BF, D, KS>>(nb);
+            if (nb >= (int64_t)4 * grid) {
+                ProfScope prof(ENATTEN_KERNEL_FWD, "fwd2_mfma", st);
+                hipLaunchKernelGGL((fwd2_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
+                                   tiles_c, (int)nb);
                 return check_launch("enatten2d_fwd");
             }
         }
