@@ -189,8 +189,43 @@ struct Geo {
     // multiple of 32 like the padded 14 * 14 would be, so no work is added, and the
     // token -> (row, column) arithmetic becomes shifts (divisions by 14 cost the
     // k = 11 kernels more registers than they have).
+    // A 10- or 12-wide halo (k = 7, 9) is numbered in two blocks instead: its first 8
+    // columns row-major, 8 per row, then the remaining 2 or 4 columns row-major.  The
+    // first block ends on a multiple of 16 tokens, so for every 16-token tile the
+    // (row, column) of a token is shifts and masks of its number (tok_rc): divisions by
+    // 10 or 12 cost those kernels up to 80 registers of hoisted quotients.
     static constexpr int SWC = SW == 14 ? 16 : SW;
+    static constexpr int W1 = (SW == 10 || SW == 12) ? 8 : 0;
     static constexpr int NK = SW * SWC;           // token numbers per wave (some unused)
+    // (row, column) in the wave's halo of token tile * 16 + x, x in [0, 16); false: no
+    // such token.  `tile` is a compile-time constant wherever this is called.
+    static __device__ __forceinline__ bool tok_rc(int tile, int x, int &r, int &c) {
+        if constexpr (W1 != 0) {
+            constexpr int A_TILES = SW * W1 / 16, W2 = SW - W1;
+            if (tile < A_TILES) {
+                const int tk = tile * 16 + x;
+                r = tk >> 3;
+                c = tk & 7;
+                return true;
+            }
+            const int tb = (tile - A_TILES) * 16 + x;
+            r = tb / W2;
+            c = W1 + tb % W2;
+            return r < SW;
+        } else {
+            const int tk = tile * 16 + x;
+            r = tk / SWC;
+            c = tk % SWC;
+            return tk < NK && c < SW;
+        }
+    }
+    // token tile * 16 + x lies in the k x k window that starts at (dr, dc) of the halo
+    template <int K>
+    static __device__ __forceinline__ bool tok_in(int tile, int x, int dr, int dc) {
+        int r, c;
+        const bool ok = tok_rc(tile, x, r, c);
+        return ok && (unsigned)(r - dr) < (unsigned)K && (unsigned)(c - dc) < (unsigned)K;
+    }
     static constexpr int NKP = (NK + 31) / 32 * 32;
     static constexpr int MT = NKP / 16;           // 16-token MFMA row tiles
     static constexpr int KSTEPS = NKP / 32;       // reduction steps of the second product
@@ -254,20 +289,21 @@ struct Geo {
     // waves per SIMD to budget registers for: one per workgroup that LDS admits
     // on a CU (a workgroup puts one wave on each of the four SIMDs), at most 2
     static constexpr int WAVES = NW == 4 && SP == 1 ? (2 * LDS_BYTES <= 160 * 1024 ? 2 : 1) : 2;
-    // staged LDS row of wave token tk whose halo starts at (orow, ocol) of the
+    // staged LDS row of wave token tile * 16 + x whose halo starts at (orow, ocol) of the
     // staged block; numbers that are no token read the all-zero row
-    static __device__ __forceinline__ int token_row(int tk, int orow, int ocol) {
-        const int r = tk / SWC, c = tk % SWC;
-        return (tk < NK && c < SW) ? (orow + r) * HC + ocol + c : (int)ZROW;
+    static __device__ __forceinline__ int token_row(int tile, int x, int orow, int ocol) {
+        int r, c;
+        return tok_rc(tile, x, r, c) ? (orow + r) * HC + ocol + c : (int)ZROW;
     }
     // the same when the rows of the staged block are kept in LDS cyclically: image
     // row y of the block sits in row slot y % HR, and rot = (first image row of the
     // block) % HR
-    static __device__ __forceinline__ int token_row_rot(int tk, int orow, int ocol, int rot) {
-        const int r = tk / SWC, c = tk % SWC;
-        int x = orow + r + rot;
-        x = x >= HR ? x - HR : x;
-        return (tk < NK && c < SW) ? x * HC + ocol + c : (int)ZROW;
+    static __device__ __forceinline__ int token_row_rot(int tile, int x, int orow, int ocol, int rot) {
+        int r, c;
+        const bool ok = tok_rc(tile, x, r, c);
+        int y = orow + r + rot;
+        y = y >= HR ? y - HR : y;
+        return ok ? y * HC + ocol + c : (int)ZROW;
     }
 };
 

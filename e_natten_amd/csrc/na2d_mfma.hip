@@ -104,8 +104,8 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
             prefetch(nxt, lqn, y0, nr);
         }
         const int rot = ROLL ? lq.hr0 % G::HR : 0;
-        auto trow = [&](int tk) __attribute__((always_inline)) {
-            return ROLL ? G::token_row_rot(tk, lq.orow, lq.ocol, rot) : G::token_row(tk, lq.orow, lq.ocol);
+        auto trow = [&](int tile, int x) __attribute__((always_inline)) {
+            return ROLL ? G::token_row_rot(tile, x, lq.orow, lq.ocol, rot) : G::token_row(tile, x, lq.orow, lq.ocol);
         };
 
         if (lq.wave_on) {
@@ -114,18 +114,14 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
             float mx = -INFINITY;
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
-                const int kk = mt * 16 + n;
-                const typename G::ARow kp = G::a_row(lds_k, trow(kk), g);
+                const typename G::ARow kp = G::a_row(lds_k, trow(mt, n), g);
                 f32x4 c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ds = 0; ds < G::DS; ds++)
                     c = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(kp, ds)), qreg[ds], c);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int tk = mt * 16 + g * 4 + i;  // halo token of accumulator row g*4+i
-                    const int kr = tk / G::SWC, kc = tk % G::SWC;
-                    const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
-                                    (unsigned)(kc - lq.dc) < (unsigned)KS;
+                    const bool ok = G::template tok_in<KS>(mt, g * 4 + i, lq.dr, lq.dc);
                     c[i] = ok ? c[i] * sc2 : -INFINITY;
                     mx = fmaxf(mx, c[i]);
                 }
@@ -154,7 +150,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
                 typename G::TRow vp[2];
 #pragma unroll
                 for (int h = 0; h < 2; h++)
-                    vp[h] = G::t_row(lds_v, trow(ks * 32 + h * 16 + g * 4 + (n >> 2)), n);
+                    vp[h] = G::t_row(lds_v, trow(ks * 2 + h, g * 4 + (n >> 2)), n);
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++)
                     o[mt] = mfma16<BF>(
@@ -215,24 +211,21 @@ __global__ __launch_bounds__(256, 2) void fwd2_mfma(FwdArgs a, int tiles_r, int 
         for (int ds = 0; ds < G::DS; ds++) qreg[ds] = qnext[ds];
         __syncthreads();
         fetch_rows(a.v, cur, lq);
-        auto trow = [&](int tk) __attribute__((always_inline)) { return G::token_row(tk, lq.orow, lq.ocol); };
+        auto trow = [&](int tile, int x) __attribute__((always_inline)) { return G::token_row(tile, x, lq.orow, lq.ocol); };
         s16x8 pb[G::KSTEPS];
         float mx = -INFINITY, sum = 0.f;
         if (lq.wave_on) {
             f32x4 acc[G::MT];
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
-                const typename G::ARow kp = G::a_row(lds_x, trow(mt * 16 + n), g);
+                const typename G::ARow kp = G::a_row(lds_x, trow(mt, n), g);
                 f32x4 c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ds = 0; ds < G::DS; ds++)
                     c = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(kp, ds)), qreg[ds], c);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int tk = mt * 16 + g * 4 + i;
-                    const int kr = tk / G::SWC, kc = tk % G::SWC;
-                    const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
-                                    (unsigned)(kc - lq.dc) < (unsigned)KS;
+                    const bool ok = G::template tok_in<KS>(mt, g * 4 + i, lq.dr, lq.dc);
                     c[i] = ok ? c[i] * sc2 : -INFINITY;
                     mx = fmaxf(mx, c[i]);
                 }
@@ -272,7 +265,7 @@ __global__ __launch_bounds__(256, 2) void fwd2_mfma(FwdArgs a, int tiles_r, int 
                 typename G::TRow vp[2];
 #pragma unroll
                 for (int h = 0; h < 2; h++)
-                    vp[h] = G::t_row(lds_x, trow(ks * 32 + h * 16 + g * 4 + (n >> 2)), n);
+                    vp[h] = G::t_row(lds_x, trow(ks * 2 + h, g * 4 + (n >> 2)), n);
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++)
                     o[mt] = mfma16<BF>(
@@ -300,8 +293,14 @@ __global__ __launch_bounds__(256, 2) void fwd2_mfma(FwdArgs a, int tiles_r, int 
 // Per-query math: e_natten/triton.py:383-398.
 // FRAME: walk only the tiles of the frame of `ts` (the inner tiles are served by
 // the fused backward).
+// head_dim 32 with kernel_size 7 and 9: the dQ pass fits the 168 registers of three waves
+// per SIMD (LDS admits three workgroups per CU and more); B8 N2 112x112 k = 7: 27.8 -> 24.4
+// us, B4 N4 128x128 k = 9: 37.1 -> 35.0.  The forward is as fast or faster compiled for two
+// (it then takes about 150 registers and runs three per SIMD anyway).
+template <int D, int KS, int NW>
+constexpr int kDqWaves = D == 32 && (KS == 7 || KS == 9) && NW == 4 ? 3 : Geo<D, KS, NW>::WAVES;
 template <bool BF, int D, int KS, bool FRAME, bool ROLL, int NW = 4>
-__global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void bwd_dq_mfma(BwdArgs a, TileSet ts, int ntiles, Runs rp) {
+__global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void bwd_dq_mfma(BwdArgs a, TileSet ts, int ntiles, Runs rp) {
     using G = Geo<D, KS, NW>;
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
@@ -380,8 +379,8 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
             prefetch(nxt, lqn, y0, nr);
         }
         const int rot = ROLL ? lq.hr0 % G::HR : 0;
-        auto trow = [&](int tk) __attribute__((always_inline)) {
-            return ROLL ? G::token_row_rot(tk, lq.orow, lq.ocol, rot) : G::token_row(tk, lq.orow, lq.ocol);
+        auto trow = [&](int tile, int x) __attribute__((always_inline)) {
+            return ROLL ? G::token_row_rot(tile, x, lq.orow, lq.ocol, rot) : G::token_row(tile, x, lq.orow, lq.ocol);
         };
 
         if (lq.wave_on) {
@@ -398,8 +397,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
             float dpart = 0.f;
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
-                const int kk = mt * 16 + n;
-                const int row = trow(kk);
+                const int row = trow(mt, n);
                 const typename G::ARow kp = G::a_row(lds_k, row, g), vp = G::a_row(lds_v, row, g);
                 f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -409,10 +407,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
                 }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int tk = mt * 16 + g * 4 + i;
-                    const int kr = tk / G::SWC, kc = tk % G::SWC;
-                    const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
-                                    (unsigned)(kc - lq.dc) < (unsigned)KS;
+                    const bool ok = G::template tok_in<KS>(mt, g * 4 + i, lq.dr, lq.dc);
                     cs[i] = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - lse2 : -INFINITY);
                     dpart = fmaf(cs[i], cp[i], dpart);
                     dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(cs[i]);
@@ -426,7 +421,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
                 if constexpr (kKeepDp) {
                     cp = dp[mt];
                 } else {
-                    const typename G::ARow vp = G::a_row(lds_v, trow(mt * 16 + n), g);
+                    const typename G::ARow vp = G::a_row(lds_v, trow(mt, n), g);
                     cp = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int ds = 0; ds < G::DS; ds++)
@@ -447,7 +442,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
                 typename G::TRow kp[2];
 #pragma unroll
                 for (int h = 0; h < 2; h++)
-                    kp[h] = G::t_row(lds_k, trow(ks * 32 + h * 16 + g * 4 + (n >> 2)), n);
+                    kp[h] = G::t_row(lds_k, trow(ks * 2 + h, g * 4 + (n >> 2)), n);
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++)
                     dq[mt] = mfma16<BF>(
@@ -520,13 +515,13 @@ __global__ __launch_bounds__(256, 2) void bwd_dq2_mfma(BwdArgs a, TileSet ts, in
         __syncthreads();
         fetch_rows(a.k, cur, lq);
         fetch_q(cur, lq);
-        auto trow = [&](int tk) __attribute__((always_inline)) { return G::token_row(tk, lq.orow, lq.ocol); };
+        auto trow = [&](int tile, int x) __attribute__((always_inline)) { return G::token_row(tile, x, lq.orow, lq.ocol); };
 
         f32x4 dp[G::MT];
         if (lq.wave_on) {
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
-                const typename G::ARow vp = G::a_row(lds_x, trow(mt * 16 + n), g);
+                const typename G::ARow vp = G::a_row(lds_x, trow(mt, n), g);
                 f32x4 cp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ds = 0; ds < G::DS; ds++)
@@ -554,17 +549,14 @@ __global__ __launch_bounds__(256, 2) void bwd_dq2_mfma(BwdArgs a, TileSet ts, in
             float dpart = 0.f;
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
-                const typename G::ARow kp = G::a_row(lds_x, trow(mt * 16 + n), g);
+                const typename G::ARow kp = G::a_row(lds_x, trow(mt, n), g);
                 f32x4 cs = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ds = 0; ds < G::DS; ds++)
                     cs = mfma16<BF>(*reinterpret_cast<const s16x8 *>(G::a_at(kp, ds)), qreg[ds], cs);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int tk = mt * 16 + g * 4 + i;
-                    const int kr = tk / G::SWC, kc = tk % G::SWC;
-                    const bool ok = tk < G::NK && (unsigned)(kr - lq.dr) < (unsigned)KS &&
-                                    (unsigned)(kc - lq.dc) < (unsigned)KS;
+                    const bool ok = G::template tok_in<KS>(mt, g * 4 + i, lq.dr, lq.dc);
                     const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - lse2 : -INFINITY);
                     dpart = fmaf(p, dp[mt][i], dpart);
                     dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p);
@@ -586,7 +578,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq2_mfma(BwdArgs a, TileSet ts, in
                 typename G::TRow kp[2];
 #pragma unroll
                 for (int h = 0; h < 2; h++)
-                    kp[h] = G::t_row(lds_x, trow(ks * 32 + h * 16 + g * 4 + (n >> 2)), n);
+                    kp[h] = G::t_row(lds_x, trow(ks * 2 + h, g * 4 + (n >> 2)), n);
 #pragma unroll
                 for (int mt = 0; mt < G::DT; mt++)
                     dq[mt] = mfma16<BF>(
@@ -666,8 +658,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
     const float sc2 = s.scale * kLog2e;
     const int orow = (wave >> 1) * 4, ocol = (wave & 1) * 4;
     int rot = 0;  // ROLL: (first image row of the staged block) % HR
-    auto row_of = [&](int tk) __attribute__((always_inline)) {
-        return ROLL ? G::token_row_rot(tk, orow, ocol, rot) : G::token_row(tk, orow, ocol);
+    auto row_of = [&](int tile, int x) __attribute__((always_inline)) {
+        return ROLL ? G::token_row_rot(tile, x, orow, ocol, rot) : G::token_row(tile, x, orow, ocol);
     };
     auto pick = [&](int t) __attribute__((always_inline)) {
         return ROLL ? inner_tile_cm(t, ts, s.N) : inner_tile(t, ts, s.N);
@@ -773,7 +765,7 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
 #pragma unroll
             for (int m2 = 0; m2 < 2; m2++) {
                 const int mt = ks * 2 + m2;
-                const int row = row_of(mt * 16 + n);
+                const int row = row_of(mt, n);
                 const typename G::ARow qp = G::a_row(lds_q, row, g), gp = G::a_row(lds_g, row, g);
                 f32x4 cs = {0.f, 0.f, 0.f, 0.f}, cp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -783,11 +775,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
                 }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int tk = mt * 16 + g * 4 + i;  // query of accumulator row g*4+i
-                    const float2 st = lds_stat[row_of(tk)];
-                    const bool ok = tk < G::NK &&
-                                    (unsigned)(tk / G::SWC - (n >> 2)) < (unsigned)KS &&
-                                    (unsigned)(tk % G::SWC - (n & 3)) < (unsigned)KS;
+                    const float2 st = lds_stat[row_of(mt, g * 4 + i)];  // query of accumulator row g*4+i
+                    const bool ok = G::template tok_in<KS>(mt, g * 4 + i, n >> 2, n & 3);
                     const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
                     pb[m2 * 4 + i] = cvt16<BF>(p);
                     dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
@@ -796,7 +785,7 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
             typename G::TRow qt[2], gt[2];
 #pragma unroll
             for (int h = 0; h < 2; h++) {
-                const int row = row_of(ks * 32 + h * 16 + g * 4 + (n >> 2));
+                const int row = row_of(ks * 2 + h, g * 4 + (n >> 2));
                 qt[h] = G::t_row(lds_q, row, n);
                 gt[h] = G::t_row(lds_g, row, n);
             }
@@ -1153,23 +1142,19 @@ constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= 11;
 
 // The dQ pass with one halo in LDS at a time (bwd_dq2_mfma): where two halos leave LDS for
 // one workgroup per CU, one halo fits twice, and the 16x8 tiles are not used.  head_dim 64
-// (kernel_size 13): 96 -> 79 us at B2 N8 128x128.  At head_dim 128 (kernel_size 7 and 9) it
-// needs more registers than a wave has at two per SIMD (40-50 spilled) and was measured
-// slower (112 -> 162 us, 125 -> 155 us), so it is not built there.
+// (kernel_size 13): 96 -> 79 us at B2 N8 128x128.  head_dim 128 (kernel_size 7 and 9), B4 N4
+// 128x128: 110.6 -> 72.2 us and 123.8 -> 80.3; B8 N8: 431 -> 302; B2 N2 64x64: 10.9 -> 10.1.
 template <int D, int KS>
-constexpr bool kDq2Built = D == 64 && Geo<D, KS>::WAVES == 1 && !kTallDqBuilt<D, KS> &&
+constexpr bool kDq2Built = (D == 64 || D == 128) && Geo<D, KS>::WAVES == 1 && !kTallDqBuilt<D, KS> &&
                            2 * (Geo<D, KS>::ROWS * Geo<D, KS>::PITCH * 2 + 1024) <= 160 * 1024;
 
-// The dK/dV pass with two waves per 4x4 block of keys, each on half of the block's
-// queries (Geo's SP): where the staged queries leave LDS for one workgroup per CU, a
-// SIMD then still holds two waves.  Built for head_dim 64 (the partial sums of the
-// second wave pass through 32 KB of LDS there).
 // The forward with one halo in LDS at a time (fwd2_mfma), for head_dim 128 where two halos
-// leave LDS for one workgroup per CU (kernel_size 7 and 9).  It pays from four tiles per
-// workgroup of its grid on (us, fwd_mfma -> fwd2_mfma, bf16, 128x128 images): k = 7
-// B2 N4 48.6 -> 44.2, B4 N4 91.8 -> 84.4, B8 N8 364 -> 353; k = 9 B2 N4 56.6 -> 54.2,
-// B4 N4 106.6 -> 103.0; with fewer tiles the walk down the columns of fwd_mfma, or its
-// single workgroup per CU, is as fast or faster (B1 N2: 14.8 -> 16.3).
+// leave LDS for one workgroup per CU (kernel_size 7 and 9).  Launched where the tiles give
+// every CU its two workgroups (us, fwd_mfma -> fwd2_mfma, bf16, 128x128 images): k = 7
+// B1 N2 14.1 -> 12.5, B1 N4 26.3 -> 20.3, B4 N4 91.8 -> 60.5, B8 N8 364 -> 245; k = 9
+// B1 N4 28.0 -> 22.4, B4 N4 106.6 -> 68.5.  With fewer tiles fwd_mfma's single workgroup
+// per CU is faster (B2 N2 64x64: 9.3 us against 9.9).  At head_dim 64 (kernel_size 11, 13)
+// the 16x8 tiles of fwd_mfma are faster (57.8 us against 59.3, 61.6 against 69.5).
 template <int D, int KS>
 constexpr bool kFwd2Built = D == 128 && Geo<D, KS>::WAVES == 1 &&
                             2 * (Geo<D, KS>::ROWS * Geo<D, KS>::PITCH * 2 + 1024) <= 160 * 1024;
@@ -1197,7 +1182,7 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
         }
         if constexpr (kFwd2Built<D, KS>) {
             const int grid = persistent_grid<fwd2_mfma<BF, D, KS>>(nb);
-            if (nb >= (int64_t)4 * grid) {
+            if (nb >= 2 * 256) {  // two workgroups for each of the 256 CUs
                 ProfScope prof(ENATTEN_KERNEL_FWD, "fwd2_mfma", st);
                 hipLaunchKernelGGL((fwd2_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
                                    tiles_c, (int)nb);

@@ -121,20 +121,18 @@ def test_config3_fp32_readme_shape(side):
     _case((4, 4, side, side, 128), F32, 5, what="C3 side %d" % side)
 
 
-@pytest.mark.parametrize("shape,ks,dtype", [((2, 4, 128, 128, 128), 7, BF), ((1, 8, 124, 140, 128), 9, torch.float16)])
-def test_forward_with_one_halo_in_lds_at_a_time(shape, ks, dtype, _lib):
-    # head_dim 128 with kernel_size 7 and 9, from four tiles per workgroup on (2048 and
-    # 2304 tiles of 8x8 here): the forward stages K, then V over it.  Straight through the C ABI
-    # into NaN-filled buffers, O and the log-sum-exp against the C oracle's forward.
-    from oracle import na2d_c
+@pytest.mark.parametrize("shape,ks,dtype", [((2, 4, 128, 128, 128), 7, BF), ((1, 8, 124, 140, 128), 9, torch.float16),
+                                            ((1, 2, 128, 128, 128), 7, BF), ((8, 2, 112, 112, 32), 7, BF)])
+def test_one_halo_in_lds_at_a_time(shape, ks, dtype, _lib):
+    # head_dim 128 with kernel_size 7 and 9: the forward (from 512 tiles of 8x8 on; the
+    # third shape has exactly 512) and the dQ pass stage K and V in turn in one buffer.
+    # The last shape is the dQ pass of head_dim 32 compiled for three waves per SIMD.
+    # Straight through the C ABI into NaN-filled buffers, against the C oracle.
     q, k, v, g = make_inputs(shape, dtype, 21)
-    o, lse = run_capi(q, k, v, g, ks)[:2]
-    ro, rl = na2d_c.forward(q, k, v, ks, 1.0)
-    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
-    err = (o.float() - ro.float()).abs().max().item() / ro.float().abs().max().item()
-    print("   fwd2 %s k%d rel err %.3e" % (shape, ks, err), flush=True)
-    assert err <= 2e-2
-    assert (lse - rl).abs().max().item() <= 2e-2
+    o, lse, dq, dk, dv = run_capi(q, k, v, g, ks)
+    ref = oracle_all(q, k, v, g, ks)
+    assert_close((o, dq, dk, dv), (ref[0], ref[2], ref[3], ref[4]), dtype, "one halo %s k%d" % (shape, ks))
+    assert torch.isfinite(lse).all() and (lse - ref[1]).abs().max().item() <= 2e-2
 
 
 def test_config4_large_window(path):
@@ -164,6 +162,10 @@ def test_config5_backbone_stages(heads, side, path):
     ((2, 2, 12, 12, 32), 1, BF),     # k = 1: O == V
     ((1, 2, 20, 18, 64), 5, F16),
     ((1, 2, 20, 18, 128), 7, F16),
+    ((1, 2, 21, 35, 128), 7, BF),    # one halo in LDS at a time (dQ pass), ragged sides
+    ((1, 2, 27, 20, 128), 9, F16),
+    ((2, 2, 19, 30, 32), 7, BF),     # halo tokens numbered in two blocks (10 and 12 wide)
+    ((1, 2, 25, 33, 32), 9, F16),
     ((1, 3, 11, 12, 3), 3, F32),     # odd head dims: scalar loads
     ((1, 1, 9, 9, 5), 5, BF),
     ((1, 1, 10, 9, 48), 3, BF),
