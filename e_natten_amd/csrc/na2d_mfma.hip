@@ -1130,19 +1130,21 @@ bool roll_pays(int64_t ntiles, int grid) {
 // per pixel, and at k = 11 and 13, where the halo of an 8x8 tile leaves LDS for one
 // workgroup per CU, two waves per SIMD instead of one.  Measured at B4 N4 128x128
 // (8x8 -> 16x8, us): forward 40 -> 39 (k=7), 76 -> 53 (k=11), 82 -> 55 (k=13); dQ pass
-// 59 -> 48 (k=7), 82 -> 59 (k=9), 92 -> 65 (k=11).  Not used where it was measured
-// slower or no faster: k <= 5, head_dim 32, and the dQ pass at k = 13, which does not
-// fit the 256 registers a wave has at two waves per SIMD (it spills: 95 -> 118 us).
+// 59 -> 48 (k=7), 82 -> 59 (k=9).  Not used where it was measured slower or no faster:
+// k <= 5, head_dim 32, and the dQ pass at k = 11 and 13, where the pass with one halo in
+// LDS at a time (bwd_dq2_mfma) is faster (k = 11: 87 us against 75; at k = 13 the 16x8
+// tiles spill).
 template <int D, int KS>
 constexpr bool kTallBuilt =
     D == 64 && KS >= 7 &&
     (size_t)2 * Geo<D, KS, 8>::ROWS * Geo<D, KS, 8>::PITCH * sizeof(short) <= 160 * 1024;
 template <int D, int KS>
-constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= 11;
+constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= 9;
 
 // The dQ pass with one halo in LDS at a time (bwd_dq2_mfma): where two halos leave LDS for
 // one workgroup per CU, one halo fits twice, and the 16x8 tiles are not used.  head_dim 64
-// (kernel_size 13): 96 -> 79 us at B2 N8 128x128.  head_dim 128 (kernel_size 7 and 9), B4 N4
+// (kernel_size 11 and 13): 96 -> 79 us at B2 N8 128x128 k = 13; k = 11, against the 16x8
+// tiles: 87.3 -> 75.2 us at B4 N4 128x128, 380 -> 296 at 256x256, 27.0 -> 23.1 at B2 N8 64x64.  head_dim 128 (kernel_size 7 and 9), B4 N4
 // 128x128: 110.6 -> 72.2 us and 123.8 -> 80.3; B8 N8: 431 -> 302; B2 N2 64x64: 10.9 -> 10.1.
 template <int D, int KS>
 constexpr bool kDq2Built = (D == 64 || D == 128) && Geo<D, KS>::WAVES == 1 && !kTallDqBuilt<D, KS> &&

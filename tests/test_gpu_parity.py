@@ -95,7 +95,7 @@ def test_fused_backward_path(shape, dtype, _lib):
     ((6, 7, 56, 56, 64), 7, BF),      # row-major walk (head_dim below 128), 16x8 tiles
     ((4, 8, 40, 72, 64), 9, BF),      # 16x8 tiles, last tile row half outside the image
     ((8, 8, 72, 40, 64), 13, BF),     # 16x8 tiles of eight waves (forward), ragged last tile row
-    ((4, 8, 56, 88, 64), 11, F16),    # 16x8 tiles in the forward and the dQ pass
+    ((4, 8, 56, 88, 64), 11, F16),    # 16x8 tiles in the forward, one-halo dQ pass
     ((2, 3, 33, 47, 128), 5, BF),     # ragged sides
     ((2, 2, 24, 40, 48), 5, F32),     # general kernels
 ])
