@@ -412,6 +412,36 @@ def test_deterministic_bitwise(path):
         assert torch.equal(x, y)
 
 
+@pytest.mark.parametrize("dtype", [BF, F32])
+def test_tensors_beyond_2_31_elements(dtype, _lib):
+    # 66 x 16 images of 128 x 128 x 128: 2.2e9 elements per tensor, so the element offset of
+    # the last images does not fit 31 bits and their byte offset not 32.  Inputs are drawn
+    # on the GPU; images at both ends and in the middle are compared with a call on a copy
+    # of that image alone (which the other tests hold against the oracle).
+    from e_natten_amd import natten2d
+    dev = torch.device("cuda:0")
+    B, N, H, W, D = 66, 16, 128, 128, 128
+    assert B * N * H * W * D > 2 ** 31
+    gen = torch.Generator(device=dev).manual_seed(5)
+    q, k, v, g = (torch.randn((B, N, H, W, D), device=dev, dtype=dtype, generator=gen) for _ in range(4))
+    q, k, v = (t.requires_grad_(True) for t in (q, k, v))
+    o = natten2d(q, k, v, 5)
+    grads = torch.autograd.grad(o, (q, k, v), g)
+    torch.cuda.synchronize()
+    for b, n in ((0, 0), (33, 7), (B - 1, N - 1)):
+        qs, ks, vs = (t[b:b + 1, n:n + 1].detach().clone().requires_grad_(True) for t in (q, k, v))
+        os_ = natten2d(qs, ks, vs, 5)
+        gs = torch.autograd.grad(os_, (qs, ks, vs), g[b:b + 1, n:n + 1].clone())
+        for name, big, small in zip(("O", "dQ", "dK", "dV"), (o,) + grads, (os_,) + gs):
+            x, r = big[b:b + 1, n:n + 1].float(), small.float()
+            assert torch.isfinite(x).all(), "%s of image (%d, %d) has non-finite values" % (name, b, n)
+            err = (x - r).abs().max().item()
+            bound = 1e-5 if dtype == F32 else 2 ** -7 * r.abs().max().item()
+            assert err <= bound, "%s of image (%d, %d): %.3e > %.3e" % (name, b, n, err, bound)
+    del q, k, v, g, o, grads
+    torch.cuda.empty_cache()
+
+
 def test_full_size_invariants():
     # properties that need no oracle, at the benchmark's full size:
     # rows of P sum to 1  => sum_keys dV == sum_queries dO

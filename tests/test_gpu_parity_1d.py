@@ -171,3 +171,30 @@ def test_rpb_1d():
         err = O.max_abs_err(x, r) / max(1.0, r.abs().max().item())
         print("   rpb 1d", name, "err %.3e" % err, flush=True)
         assert err <= FP32_MAX_ABS, (name, err)
+
+
+def test_sequences_beyond_2_31_elements(_lib):
+    # 66 x 16 sequences of 16384 x 128: 2.2e9 elements per tensor; sequences at both ends and
+    # in the middle against a call on a copy of that sequence alone
+    from e_natten_amd import natten1d
+    dev = torch.device("cuda:0")
+    B, N, T, D = 66, 16, 16384, 128
+    assert B * N * T * D > 2 ** 31
+    gen = torch.Generator(device=dev).manual_seed(6)
+    q, k, v, g = (torch.randn((B, N, T, D), device=dev, dtype=torch.bfloat16, generator=gen) for _ in range(4))
+    q, k, v = (t.requires_grad_(True) for t in (q, k, v))
+    o = natten1d(q, k, v, 13)
+    grads = torch.autograd.grad(o, (q, k, v), g)
+    torch.cuda.synchronize()
+    for b, n in ((0, 0), (33, 7), (B - 1, N - 1)):
+        qs, ks, vs = (t[b:b + 1, n:n + 1].detach().clone().requires_grad_(True) for t in (q, k, v))
+        os_ = natten1d(qs, ks, vs, 13)
+        gs = torch.autograd.grad(os_, (qs, ks, vs), g[b:b + 1, n:n + 1].clone())
+        for name, big, small in zip(("O", "dQ", "dK", "dV"), (o,) + grads, (os_,) + gs):
+            x, r = big[b:b + 1, n:n + 1].float(), small.float()
+            assert torch.isfinite(x).all()
+            err = (x - r).abs().max().item()
+            assert err <= 2 ** -7 * r.abs().max().item(), "%s of sequence (%d, %d): %.3e" % (name, b, n, err)
+    del q, k, v, g, o, grads
+    torch.cuda.empty_cache()
+
