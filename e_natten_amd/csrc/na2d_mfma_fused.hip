@@ -107,7 +107,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
         if (per % ts.tiles_r == 0 && hi - lo == per && per / ts.tiles_r >= 2 * slots) {
             deal_ncols = per / ts.tiles_r;
             deal_lo = lo;
-            sc.t = lo + slot * ts.tiles_r;  // round 0: column `slot`
+            sc.t = lo + slot * ts.tiles_r;  // r = 0: column `slot`
             seg_end = sc.t + ts.tiles_r;
             sc.t_end = hi;
         }
