@@ -1,6 +1,7 @@
 """Seeded random shapes through the C ABI against the CPU oracle: every kernel family
 (16-bit matrix-core, float32 matrix-core, 1D matrix-core, general), both backward paths,
-ragged and tile-aligned images, batch * heads from 1 to hundreds."""
+ragged and tile-aligned images, batch * heads from 1 to hundreds; rectangular and causal
+windows and the relative position bias against the dense-mask oracle."""
 import random
 
 import pytest
@@ -94,3 +95,47 @@ def _random_1d(shape, ks, dtype, seed):
             assert O.max_abs_err(x, r) <= FP32_MAX_ABS, (name, O.max_abs_err(x, r))
         else:
             assert O.rel_err(x, r) <= BF16_REL, (name, O.rel_err(x, r))
+
+
+def _cases_window(n, seed):
+    rnd = random.Random(seed)
+    out = []
+    for it in range(n):
+        D = rnd.choice([8, 32, 64, 128, 24])
+        causal = (rnd.random() < 0.4, rnd.random() < 0.4)
+        kh = rnd.choice([1, 2, 3, 4, 6, 7]) if causal[0] else rnd.choice([1, 3, 5, 7, 9])
+        kw = rnd.choice([1, 2, 3, 5, 8]) if causal[1] else rnd.choice([1, 3, 5, 7, 9])
+        H, W = rnd.randint(kh, 26), rnd.randint(kw, 26)
+        dt = rnd.choice([torch.float32, torch.bfloat16, torch.float16])
+        rpb = rnd.random() < 0.4 and not any(causal)
+        out.append(((rnd.choice([1, 2]), rnd.choice([1, 3]), H, W, D), (kh, kw), causal, dt, rpb,
+                    rnd.choice([1.0, 0.5, D ** -0.5]), it))
+    return out
+
+
+@pytest.mark.parametrize("shape,kernel,causal,dtype,with_rpb,scale,seed", _cases_window(24, 77))
+def test_random_windows(shape, kernel, causal, dtype, with_rpb, scale, seed, lib):
+    # rectangular and causal windows and the relative position bias against the dense-mask
+    # oracle (float64 autograd), forward and backward, d_rpb included
+    from e_natten_amd import natten2d
+    print("case window", shape, kernel, causal, dtype, "rpb" if with_rpb else "", flush=True)
+    q, k, v, g = make_inputs(shape, dtype, seed=1000 + seed, q_scale=1.0 if dtype == torch.float32 else 0.5)
+    rpb = None
+    if with_rpb:
+        gen = torch.Generator().manual_seed(seed)
+        rpb = torch.randn((shape[1], 2 * kernel[0] - 1, 2 * kernel[1] - 1), generator=gen).to(dtype)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    rr = rpb.double().requires_grad_(True) if with_rpb else None
+    o_ref = O.natten2d_window_dense_mask(qr, kr, vr, kernel, causal, scale, rr)
+    refs = (o_ref.detach(),) + tuple(torch.autograd.grad(o_ref, (qr, kr, vr) + ((rr,) if with_rpb else ()), g.double()))
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    rg = rpb.cuda().requires_grad_(True) if with_rpb else None
+    o = natten2d(qg, kg, vg, kernel, scale, 1, causal, rg)
+    outs = (o,) + tuple(torch.autograd.grad(o, (qg, kg, vg) + ((rg,) if with_rpb else ()), g.cuda()))
+    for name, x, r in zip(("O", "dQ", "dK", "dV", "d_rpb"), outs, refs):
+        x = x.detach().cpu()
+        assert torch.isfinite(x.float()).all(), name
+        if dtype == torch.float32:
+            assert O.max_abs_err(x, r) <= (FP32_MAX_ABS if name != "d_rpb" else 2e-3), (name, O.max_abs_err(x, r))
+        else:
+            assert O.rel_err(x, r) <= (BF16_REL if name != "d_rpb" else 3e-2), (name, O.rel_err(x, r))
