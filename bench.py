@@ -134,7 +134,20 @@ def cpu_baseline(shape, ks, dtype, useful_flop, budget_rows=8):
     na2d_c.forward(q, k, v, ks, nthreads=threads)
     na2d_c.backward(q, k, v, d_o, ks, nthreads=threads)
     c_s = time.perf_counter() - t0
+
+    # The loop port on a WHOLE configuration that it finishes in seconds, nothing scaled:
+    # the same batch, heads, head_dim and kernel_size on 32x32 images.
+    whole = None
+    if H >= 32 and W >= 32:
+        ws = (B, N, 32, 32, D)
+        wq, wk, wv, wg = (torch.randn(ws, generator=g).to(dtype).float() for _ in range(4))
+        wq, wk, wv = (t.requires_grad_(True) for t in (wq, wk, wv))
+        t0 = time.perf_counter()
+        O.natten2d_loops(wq, wk, wv, ks).backward(wg)
+        whole = {"workload": "B=%d heads=%d H=W=32 head_dim=%d kernel_size=%d, all rows" % (B, N, D, ks),
+                 "ms": (time.perf_counter() - t0) * 1e3}
     return {
+        "loop_port_whole_config": whole,
         "value": useful_flop / loops_s / 1e12, "unit": "TFLOP/s", "cores": threads,
         "kind": "port", "ms": loops_s * 1e3,
         "sample": "loop port of the reference algorithm, fp32, query/key rows %d..%d of %d "
@@ -323,7 +336,10 @@ def main():
     roofline = {
         "bound": "hbm", "kernel": kern[dom]["kernel"], "achieved": kern[dom]["GBps"],
         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": kern[dom]["GBps"] / HBM_PEAK_GBS,
-        "traffic": traffic, "kernels": kern,
+        "traffic": traffic,
+        "traffic_source": ("profiles/hbm_traffic.txt: rocprofv3 FETCH_SIZE + WRITE_SIZE of an earlier run "
+                           "of this workload, not counted in this run") if traffic else None,
+        "kernels": kern,
         "path_alg_bytes": alg["path"], "path_kernel_ms": kernel_ms,
         "path_GBps": alg["path"] / (kernel_ms * 1e-3) / 1e9,
         "path_frac": alg["path"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -426,6 +442,10 @@ def main():
         cb["gpu_speedup"] = cb["ms"] / ms_step
         cb["gpu_speedup_vs_vectorised_gather"] = cb["vectorised_gather_ms"] / ms_step
         cb["gpu_speedup_vs_c_openmp"] = cb["c_openmp_ms"] / ms_step
+        row32 = [r for r in out.get("sweep", []) if r["side"] == 32 and "ms_per_step" in r]
+        if cb["loop_port_whole_config"] and row32 and not args.seq:
+            cb["loop_port_whole_config"]["gpu_ms"] = row32[0]["ms_per_step"]
+            cb["loop_port_whole_config"]["gpu_speedup"] = cb["loop_port_whole_config"]["ms"] / row32[0]["ms_per_step"]
         out["cpu_baseline"] = cb
     print(json.dumps(out))
 

@@ -126,11 +126,17 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o,
  * the workspace: the two float32 per query live in a device array that is part of
  * this library (8 MiB on every GPU the library runs on, held until the process ends),
  * so calls of at most ENATTEN_STATIC_BWD_MAX_QUERIES = B * heads * H * W queries are
- * served and larger ones return ENATTEN_EUNSUPPORTED.  (float32 calls whose matrix-core
- * backward would need more of it than the array holds run on the general kernels.)  The call allocates and frees
- * nothing.  The stream's device must be the current device.  All calls on one GPU
+ * served and larger ones return ENATTEN_EUNSUPPORTED.  float32 calls run the matrix-core
+ * backward with the array as its P / dS buffers while B * heads * H * W * 2 * kernel_size^2
+ * floats fit the array's 2^21, and the general kernels beyond that.  The call allocates and
+ * frees nothing.  The stream's device must be the current device.  All calls on one GPU
  * share the one array: calls that may overlap there (different streams, different
  * threads) race; order them.
+ * Under stream capture: make one call on the device OUTSIDE capture first.  The first call on
+ * a device looks up the array's address (hipGetSymbolAddress, which may load the code object
+ * that backs the array) and the first call of every kernel family asks the runtime for the
+ * kernel's occupancy; neither is promised to be legal, or free of allocations, while a
+ * stream is capturing.  Later calls of the same family only launch kernels.
  */
 #define ENATTEN_STATIC_BWD_MAX_QUERIES (1 << 20)
 int enatten2d_bwd_static(const void *q, const void *k, const void *v, const void *o,
