@@ -123,4 +123,10 @@ bool fused_bwd_supported(const BwdArgs &a);
 int launch_bwd_fused(const BwdArgs &a, bool bf16, const TileSet &ts, int64_t ntiles,
                      hipStream_t st);
 
+// one-pass backward of the configurations whose block of all four inputs fits LDS twice
+// per CU (head_dim 32 with kernel_size <= 7, head_dim 64 with kernel_size 3)
+bool onepass_bwd_supported(const BwdArgs &a);
+int launch_bwd_onepass(const BwdArgs &a, bool bf16, const TileSet &ts, int64_t ntiles,
+                       hipStream_t st);
+
 }  // namespace enatten

@@ -172,14 +172,28 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
     }
 }
 
+// Two halos of an 8x8 tile fit LDS (the kernels that keep K and V, or Q and dO, side by side)
+template <int D, int KS>
+constexpr bool fits() {
+    return Geo<D, KS>::LDS_BYTES <= 160 * 1024;
+}
+// Workgroups per CU of the kernels that keep ONE halo in LDS at a time: two where that halo
+// fits twice, one for the largest halos (head_dim 128 with kernel_size 11 and 13: 88 and
+// 109 KB), where these kernels are the only matrix-core ones that fit at all.
+template <int D, int KS>
+constexpr int kOneHaloWgs = 2 * (Geo<D, KS>::ROWS * Geo<D, KS>::PITCH * 2 + 1024) <= 160 * 1024 ? 2 : 1;
+template <int D, int KS>
+constexpr bool kOneHaloFits = Geo<D, KS>::ROWS * Geo<D, KS>::PITCH * 2 + 1024 <= 160 * 1024;
+
 // ------------------------------------------------------------------ forward, one halo in LDS at a time
 // The forward for halos of which LDS holds two only once per CU (head_dim 128 with
-// kernel_size 7 and 9), like bwd_dq2_mfma: K rows first (logits, softmax; P stays in
-// registers as 16-bit values) while the tile's V rows are in flight, V over K behind a
-// barrier, then O^T = V^T P^T while the next tile's K rows are in flight.  Two workgroups
-// per CU, four barriers per tile; 8x8 tiles, no column walk.
+// kernel_size 7 and 9) or not at all (kernel_size 11 and 13), like bwd_dq2_mfma: K rows first
+// (logits, softmax; P stays in registers as 16-bit values) while the tile's V rows are in
+// flight, V over K behind a barrier, then O^T = V^T P^T while the next tile's K rows are in
+// flight.  Two workgroups per CU (one at kernel_size 11 and 13), four barriers per tile; 8x8
+// tiles, no column walk.
 template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256, 2) void fwd2_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles) {
+__global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void fwd2_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_x[G::ROWS * G::PITCH];
     const Shape &s = a.s;
@@ -472,7 +486,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void b
 //            the next tile's V rows are in flight meanwhile.
 // Four barriers per tile instead of two; 8x8 tiles, no column walk.
 template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256, 2) void bwd_dq2_mfma(BwdArgs a, TileSet ts, int ntiles) {
+__global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void bwd_dq2_mfma(BwdArgs a, TileSet ts, int ntiles) {
     using G = Geo<D, KS>;
     __shared__ __attribute__((aligned(16))) short lds_x[G::ROWS * G::PITCH];
     const Shape &s = a.s;
@@ -1060,10 +1074,16 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 // the forward and the dQ pass spill under that budget and get slower).
 // Size of the frame body's blocks as a kernel size (see dkdv_frame): larger than KS where the
 // pass has one workgroup per CU anyway (two parts per block) and LDS has the room.
+// Where not even one workgroup's Q and dO halos fit LDS (head_dim 128 with kernel_size 11 and
+// 13), the pass has no inner body: EVERY tile is walked by the frame body in blocks of 12x12
+// queries (78 KB for both tensors, two workgroups per CU), four to nine blocks per tile.
+template <int D, int KS>
+constexpr bool kDkdvFrameOnly = !fits<D, KS>();
 template <int D, int KS, int SP>
-constexpr int kFrameKS = SP == 2 && KS >= 9 ? 9 + KS / 2 : KS;
+constexpr int kFrameKS = kDkdvFrameOnly<D, KS> ? 5 : SP == 2 && KS >= 9 ? 9 + KS / 2 : KS;
 template <int D, int KS, int SP>
 constexpr int kDkdvWaves =
+    kDkdvFrameOnly<D, KS> ? 2 :
     SP == 1 && D <= 64 && 3 * (Geo<D, KS>::LDS_BYTES + 2048) <= 160 * 1024 ? 3 : Geo<D, KS, 4, SP>::WAVES;
 template <bool BF, int D, int KS, bool ROLL, int SP = 1>
 __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) void bwd_dkdv_mfma(
@@ -1074,29 +1094,34 @@ __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) v
     // (lse * log2e, delta) per staged query, and with two parts per block the second part's
     // partial dK and dV.  Where the frame body stages larger blocks, its partial sums lie
     // over its Q rows.
-    constexpr bool RED_OVER = !std::is_same<FG, G>::value;
+    constexpr bool FRAME_ONLY = kDkdvFrameOnly<D, KS>;
+    constexpr bool RED_OVER = !std::is_same<FG, G>::value && !FRAME_ONLY;
     constexpr size_t RED = SP > 1 ? (size_t)2 * G::DT * 256 * sizeof(f32x4) : 0;
-    constexpr size_t I_ROWS = (size_t)G::ROWS * G::PITCH * sizeof(short);
+    constexpr size_t I_ROWS = FRAME_ONLY ? 0 : (size_t)G::ROWS * G::PITCH * sizeof(short);
     constexpr size_t F_ROWS = (size_t)FG::ROWS * FG::PITCH * sizeof(short);
-    constexpr size_t I_STAT = (G::ROWS * sizeof(float2) + 15) / 16 * 16;
+    constexpr size_t I_STAT = FRAME_ONLY ? 0 : (G::ROWS * sizeof(float2) + 15) / 16 * 16;
     constexpr size_t F_STAT = (FG::ROWS * sizeof(float2) + 15) / 16 * 16;
     constexpr size_t I_ALL = 2 * I_ROWS + I_STAT + RED;
     constexpr size_t F_ALL = 2 * F_ROWS + F_STAT + (RED_OVER ? 0 : RED);
     static_assert(RED <= F_ROWS || !RED_OVER, "the partial sums lie over the staged Q rows");
     __shared__ __attribute__((aligned(16))) char lds_raw[I_ALL > F_ALL ? I_ALL : F_ALL];
     static_assert(sizeof(lds_raw) <= 160 * 1024, "LDS");
-    if ((int)blockIdx.x < inner_blocks) {
-        short *lds_q = reinterpret_cast<short *>(lds_raw);
-        short *lds_g = reinterpret_cast<short *>(lds_raw + I_ROWS);
-        float2 *lds_stat = reinterpret_cast<float2 *>(lds_raw + 2 * I_ROWS);
-        f32x4 *lds_red = reinterpret_cast<f32x4 *>(lds_raw + 2 * I_ROWS + I_STAT);
-        if (SP == 1 || threadIdx.x < 256)
-            dkdv_inner<BF, D, KS, ROLL, SP, 0>(a, ts, n_inner, rp, blockIdx.x, inner_blocks, lds_q,
-                                               lds_g, lds_stat, lds_red);
-        else  // the same number of barriers as the first part
-            dkdv_inner<BF, D, KS, ROLL, SP, SP - 1>(a, ts, n_inner, rp, blockIdx.x, inner_blocks,
-                                                    lds_q, lds_g, lds_stat, lds_red);
-    } else {
+    if constexpr (!FRAME_ONLY) {
+        if ((int)blockIdx.x < inner_blocks) {
+            short *lds_q = reinterpret_cast<short *>(lds_raw);
+            short *lds_g = reinterpret_cast<short *>(lds_raw + I_ROWS);
+            float2 *lds_stat = reinterpret_cast<float2 *>(lds_raw + 2 * I_ROWS);
+            f32x4 *lds_red = reinterpret_cast<f32x4 *>(lds_raw + 2 * I_ROWS + I_STAT);
+            if (SP == 1 || threadIdx.x < 256)
+                dkdv_inner<BF, D, KS, ROLL, SP, 0>(a, ts, n_inner, rp, blockIdx.x, inner_blocks, lds_q,
+                                                   lds_g, lds_stat, lds_red);
+            else  // the same number of barriers as the first part
+                dkdv_inner<BF, D, KS, ROLL, SP, SP - 1>(a, ts, n_inner, rp, blockIdx.x, inner_blocks,
+                                                        lds_q, lds_g, lds_stat, lds_red);
+            return;
+        }
+    }
+    {
         short *lds_q = reinterpret_cast<short *>(lds_raw);
         short *lds_g = reinterpret_cast<short *>(lds_raw + F_ROWS);
         float2 *lds_stat = reinterpret_cast<float2 *>(lds_raw + 2 * F_ROWS);
@@ -1108,11 +1133,6 @@ __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) v
 }
 
 // ------------------------------------------------------------------ dispatch
-template <int D, int KS>
-constexpr bool fits() {
-    return Geo<D, KS>::LDS_BYTES <= 160 * 1024;
-}
-
 
 // Keeping shared halo rows in LDS pays where the kernels are bound by the bytes
 // they pull through the CU's memory pipeline (d = 128) and a workgroup walks at
@@ -1148,7 +1168,7 @@ constexpr bool kTallDqBuilt = kTallBuilt<D, KS> && KS <= 9;
 // 128x128: 110.6 -> 72.2 us and 123.8 -> 80.3; B8 N8: 431 -> 302; B2 N2 64x64: 10.9 -> 10.1.
 template <int D, int KS>
 constexpr bool kDq2Built = (D == 64 || D == 128) && Geo<D, KS>::WAVES == 1 && !kTallDqBuilt<D, KS> &&
-                           2 * (Geo<D, KS>::ROWS * Geo<D, KS>::PITCH * 2 + 1024) <= 160 * 1024;
+                           kOneHaloFits<D, KS>;
 
 // The forward with one halo in LDS at a time (fwd2_mfma), for head_dim 128 where two halos
 // leave LDS for one workgroup per CU (kernel_size 7 and 9).  Launched where the tiles give
@@ -1158,15 +1178,18 @@ constexpr bool kDq2Built = (D == 64 || D == 128) && Geo<D, KS>::WAVES == 1 && !k
 // per CU is faster (B2 N2 64x64: 9.3 us against 9.9).  At head_dim 64 (kernel_size 11, 13)
 // the 16x8 tiles of fwd_mfma are faster (57.8 us against 59.3, 61.6 against 69.5).
 template <int D, int KS>
-constexpr bool kFwd2Built = D == 128 && Geo<D, KS>::WAVES == 1 &&
-                            2 * (Geo<D, KS>::ROWS * Geo<D, KS>::PITCH * 2 + 1024) <= 160 * 1024;
+constexpr bool kFwd2Built = D == 128 && Geo<D, KS>::WAVES == 1 && kOneHaloFits<D, KS>;
+// Built at all: two halos fit, or the one-halo kernels serve the forward and the dQ pass and
+// the frame body in small blocks the dK/dV pass
+template <int D, int KS>
+constexpr bool kBuilt = fits<D, KS>() || (kFwd2Built<D, KS> && kDq2Built<D, KS>);
 
 template <int D, int KS>
 constexpr int kDkdvSplit = D == 64 && Geo<D, KS>::WAVES == 1 ? 2 : 1;
 
 template <bool BF, int D, int KS>
 int fwd_launch(const FwdArgs &a, hipStream_t st) {
-    if constexpr (fits<D, KS>()) {
+    if constexpr (kBuilt<D, KS>) {
         using G = Geo<D, KS>;
         const int tiles_r = (a.s.H + G::TH - 1) / G::TH, tiles_c = (a.s.W + G::TW - 1) / G::TW;
         const int64_t nb = (int64_t)a.s.B * a.s.N * tiles_r * tiles_c;
@@ -1184,15 +1207,15 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
         }
         if constexpr (kFwd2Built<D, KS>) {
             const int grid = persistent_grid<fwd2_mfma<BF, D, KS>>(nb);
-            if (nb >= 2 * 256) {  // two workgroups for each of the 256 CUs
+            if (nb >= 2 * 256 || !fits<D, KS>()) {  // two workgroups for each of the 256 CUs
                 ProfScope prof(ENATTEN_KERNEL_FWD, "fwd2_mfma", st);
                 hipLaunchKernelGGL((fwd2_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
                                    tiles_c, (int)nb);
                 return check_launch("enatten2d_fwd");
             }
         }
-        const int grid = persistent_grid<fwd_mfma<BF, D, KS, false>>(nb);
-        {
+        if constexpr (fits<D, KS>()) {
+            const int grid = persistent_grid<fwd_mfma<BF, D, KS, false>>(nb);
             ProfScope prof(ENATTEN_KERNEL_FWD, "fwd_mfma", st);
             if (roll_pays<D>(nb, grid))
                 hipLaunchKernelGGL((fwd_mfma<BF, D, KS, kRollBuilt<D>>), dim3(grid), dim3(256), 0,
@@ -1210,7 +1233,7 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
 
 template <bool BF, int D, int KS>
 int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
-    if constexpr (fits<D, KS>()) {
+    if constexpr (kBuilt<D, KS>) {
         using G = Geo<D, KS>;
         const int tiles_r = (a.s.H + G::TH - 1) / G::TH, tiles_c = (a.s.W + G::TW - 1) / G::TW;
         const int64_t nb = (int64_t)a.s.B * a.s.N * tiles_r * tiles_c;
@@ -1219,7 +1242,7 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         ts.tiles_r = tiles_r; ts.tiles_c = tiles_c;
         ts.ir0 = (KS + 7) / 8; ts.ic0 = (KS + 7) / 8;
         ts.ni_r = (a.s.H - KS) / 8 - ts.ir0; ts.ni_c = (a.s.W - KS) / 8 - ts.ic0;
-        if (ts.ni_r <= 0 || ts.ni_c <= 0) {
+        if (ts.ni_r <= 0 || ts.ni_c <= 0 || kDkdvFrameOnly<D, KS>) {
             ts.ir0 = tiles_r; ts.ic0 = 0; ts.ni_r = 0; ts.ni_c = 0;
         }
         const int64_t slabs = (int64_t)a.s.B * a.s.N;
@@ -1230,6 +1253,22 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         // 32x32 (14.8 against 24.1) to B16 N8 128x128 (938 against 1174).
         if (path != ENATTEN_PATH_MFMA_SPLIT && fused_bwd_supported(a)) {
             const int rc = launch_bwd_fused(a, BF, ts, nb, st);
+            return rc ? rc : check_launch("enatten2d_bwd");
+        }
+
+        // The one-pass backward (head_dim 32, and 64 with kernel_size 3; na2d_mfma_onepass.hip).
+        // At these head dims the passes are bound by per-tile latency, not by HBM, so reading
+        // the inputs once only pays where the two passes are at their worst: images that are
+        // (nearly) all border tiles, which the dK/dV pass walks block by block and the one-pass
+        // kernel serves from its one staged block.  Measured, backward only, one pass vs two
+        // (us, bf16): B8 N16 14x14 d32 k7 20.4 vs 21.9; B8 N8 28x28 d32 k7 29.7 vs 33.8, k5 24.4 vs
+        // 27.4; B16 N8 16x16 d32 k3 12.2 vs 16.1; but B8 N4 40x40 d32 k7 27.9 vs 25.1 (9 of 25
+        // tiles inner), B8 N8 28x28 d64 k3 30.9 vs 26.2 (4 of 16), B8 N2 112x112 d32 k7 66 vs 54,
+        // B4 N8 128x128 d32 k5 145 vs 87.  So it is the default where at most one tile in eight
+        // is an inner tile; ENATTEN_PATH_MFMA_FUSED forces it wherever it is built.
+        if (path != ENATTEN_PATH_MFMA_SPLIT && onepass_bwd_supported(a) &&
+            (path == ENATTEN_PATH_MFMA_FUSED || 8 * n_inner <= nb)) {
+            const int rc = launch_bwd_onepass(a, BF, ts, nb, st);
             return rc ? rc : check_launch("enatten2d_bwd");
         }
 
@@ -1252,7 +1291,7 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
                 dq_done = true;
             }
         }
-        if (!dq_done) {
+        if constexpr (fits<D, KS>()) if (!dq_done) {
             const int grid = persistent_grid<bwd_dq_mfma<BF, D, KS, false, false>>(nb);
             ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq_mfma", st);
             if (roll_pays<D>(nb, grid))
@@ -1316,7 +1355,9 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
 
 bool fits_rt(int D, int ks) {
     const int rows = (8 + ks - 1) * (8 + ks - 1) + 1;
-    return (size_t)2 * rows * (D + 8) * 2 + (size_t)rows * 8 <= 160 * 1024;
+    // two halos of an 8x8 tile, or (head_dim 128) one halo for the kernels that stage one at a time
+    return (size_t)2 * rows * (D + 8) * 2 + (size_t)rows * 8 <= 160 * 1024 ||
+           (D == 128 && (size_t)rows * (D + 8) * 2 + 1024 <= 160 * 1024);
 }
 
 }  // namespace

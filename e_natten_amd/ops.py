@@ -84,7 +84,9 @@ def _check(rc: int) -> None:
         raise (ValueError if rc == 1 else RuntimeError)(msg)
 
 
-def _fwd_impl(q, k, v, kernel_size: int, scale: float):
+def _fwd_impl(q, k, v, kernel_size: int, scale: float, out=None):
+    """`out`: a view of the shape of q with unit stride on the channels that the kernels
+    write in place (the strided sub-grid of a dilated call); None allocates the output."""
     _validate(q, k, v, kernel_size)
     _require_gpu(q, "enatten::na2d_fwd")
     lib = _lib.load()
@@ -94,7 +96,7 @@ def _fwd_impl(q, k, v, kernel_size: int, scale: float):
         # like the reference's zeros_like(Q) (e_natten/triton.py:502), the output takes
         # the memory order of q: for q sliced out of a [B, H, W, 3, heads, d] projection
         # that is [B, H, W, heads, d], which the following merge of heads needs
-        o = _kernel_layout(torch.empty_like(q))
+        o = _kernel_layout(torch.empty_like(q)) if out is None else out
         lse = torch.empty((B, N, H, W), dtype=torch.float32, device=q.device)
         _check(lib.enatten2d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                  lse.data_ptr(), B, N, H, W, D, kernel_size, _DTYPES[q.dtype],
@@ -129,14 +131,14 @@ def _bwd_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
     return dq, dk, dv
 
 
-def _fwd1d_impl(q, k, v, kernel_size: int, scale: float):
+def _fwd1d_impl(q, k, v, kernel_size: int, scale: float, out=None):
     _validate(q, k, v, kernel_size, 4)
     _require_gpu(q, "enatten::na1d_fwd")
     lib = _lib.load()
     q, k, v = (_kernel_layout(t) for t in (q, k, v))
     B, N, T, D = q.shape
     with torch.cuda.device(q.device):
-        o = _kernel_layout(torch.empty_like(q))
+        o = _kernel_layout(torch.empty_like(q)) if out is None else out
         lse = torch.empty((B, N, T), dtype=torch.float32, device=q.device)
         _check(lib.enatten1d_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                  lse.data_ptr(), B, N, T, D, kernel_size, _DTYPES[q.dtype],
@@ -247,7 +249,7 @@ class Natten2dDilated(torch.autograd.Function):
     equal (x mod dilation, y mod dilation) only ever see each other, and inside such
     a sub-grid the rule is the plain one, so the operator is the undilated kernels run
     on the dilation^2 strided sub-grids of q, k, v (the C ABI takes strides), each
-    writing its own pixels of the outputs."""
+    writing its own pixels of the output in place (the C ABI takes the strides of o)."""
 
     @staticmethod
     def forward(ctx, Q, K, V, kernel_size, scale, dilation):
@@ -256,8 +258,7 @@ class Natten2dDilated(torch.autograd.Function):
         for i in range(dilation):
             for j in range(dilation):
                 sub = (slice(None), slice(None), slice(i, None, dilation), slice(j, None, dilation))
-                o_s, lse_s = torch.ops.enatten.na2d_fwd(Q[sub], K[sub], V[sub], kernel_size, scale)
-                o[sub] = o_s
+                _, lse_s = _fwd_impl(Q[sub], K[sub], V[sub], kernel_size, scale, out=o[sub])
                 lses.append(lse_s)
         ctx.save_for_backward(Q, K, V, o, *lses)
         ctx.args = (kernel_size, scale, dilation)
@@ -437,8 +438,11 @@ def natten2d(q, k, v, kernel_size=7, scale=1.0, dilation=1, is_causal=False, rpb
         return Natten2dDilated.apply(q, k, v, kernel_size, float(scale), dilation)
     if not NATIVE_BINDING:
         return Natten2d.apply(q, k, v, kernel_size, scale)
-    _validate(q, k, v, kernel_size)
-    _require_gpu(q, "natten2d")
+    # the native operator checks shapes, dtypes, devices and the kernel size itself and raises
+    # the same error classes (csrc/torch_shim.cpp: validate); only the argument's Python type
+    # is checked here, once, so that a float or a bool is not silently converted
+    if type(kernel_size) is not int:
+        raise TypeError("kernel_size must be an int")
     return torch.ops.enatten.natten2d(q, k, v, kernel_size, float(scale))
 
 
@@ -472,8 +476,7 @@ class Natten1dDilated(torch.autograd.Function):
         lses = []
         for i in range(dilation):
             sub = (slice(None), slice(None), slice(i, None, dilation))
-            o_s, lse_s = torch.ops.enatten.na1d_fwd(q[sub], k[sub], v[sub], kernel_size, scale)
-            o[sub] = o_s
+            _, lse_s = _fwd1d_impl(q[sub], k[sub], v[sub], kernel_size, scale, out=o[sub])
             lses.append(lse_s)
         ctx.save_for_backward(q, k, v, o, *lses)
         ctx.args = (kernel_size, scale, dilation)
@@ -520,8 +523,8 @@ def natten1d(q, k, v, kernel_size=7, scale=1.0, dilation=1, is_causal=False, rpb
         return Natten1dDilated.apply(q, k, v, kernel_size, float(scale), dilation)
     if not NATIVE_BINDING:
         return Natten1d.apply(q, k, v, kernel_size, scale)
-    _validate(q, k, v, kernel_size, 4)
-    _require_gpu(q, "natten1d")
+    if type(kernel_size) is not int:   # everything else is checked by the native operator
+        raise TypeError("kernel_size must be an int")
     return torch.ops.enatten.natten1d(q, k, v, kernel_size, float(scale))
 
 

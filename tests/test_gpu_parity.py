@@ -135,6 +135,77 @@ def test_one_halo_in_lds_at_a_time(shape, ks, dtype, _lib):
     assert torch.isfinite(lse).all() and (lse - ref[1]).abs().max().item() <= 2e-2
 
 
+@pytest.mark.parametrize("shape,ks,dtype", [
+    ((2, 2, 64, 64, 128), 13, BF),      # square, inner and border tiles
+    ((1, 2, 128, 128, 128), 11, BF),
+    ((1, 3, 37, 29, 128), 13, F16),     # ragged sides
+    ((2, 1, 45, 70, 128), 11, BF),
+    ((1, 2, 13, 13, 128), 13, BF),      # window = image
+    ((1, 1, 11, 40, 128), 11, F16),
+    ((1, 2, 16, 24, 128), 13, BF),      # every key within reach of a border
+])
+def test_largest_windows_at_head_dim_128(shape, ks, dtype, _lib):
+    # head_dim 128 with kernel_size 11 and 13 (the reference's own test sweeps kernel sizes up to
+    # 11, test.py:48): not even one workgroup's pair of halos fits LDS, so the forward and the
+    # dQ pass stage one halo at a time with one workgroup per CU, and the dK/dV pass walks
+    # every tile in 12x12 blocks of queries.  Through the C ABI into NaN-filled buffers.
+    from e_natten_amd import kernel_path
+    assert kernel_path(128, ks, dtype) == "mfma"
+    q, k, v, g = make_inputs(shape, dtype, 31)
+    print("case largest windows", shape, dtype, "k=%d" % ks, flush=True)
+    o, lse, dq, dk, dv = run_capi(q, k, v, g, ks)
+    ref = oracle_all(q, k, v, g, ks)
+    assert_close((o, dq, dk, dv), (ref[0], ref[2], ref[3], ref[4]), dtype, "largest windows %s k%d" % (shape, ks))
+    assert torch.isfinite(lse).all() and (lse - ref[1]).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("D,ks", [(32, 3), (32, 5), (32, 7), (64, 3)])
+@pytest.mark.parametrize("hw", [(8, 8), (8, 21), (9, 9), (13, 16), (14, 14), (15, 17), (16, 16), (23, 31),
+                                (28, 28), (40, 56), (64, 33)])
+def test_one_pass_backward_small_head_dims(D, ks, hw, _lib):
+    # The one-pass backward of head_dim 32 (kernel_size 3, 5, 7) and head_dim 64 (kernel_size 3),
+    # forced wherever it is built (automatic dispatch takes it for small calls only): images of one
+    # tile, of shifted last tiles (sides that are no multiples of 8), smaller than a staged block,
+    # and with inner tiles; against the oracle and, bit for bit in dK and dV's inputs, finite
+    # everywhere (outputs hold NaN beforehand).
+    from e_natten_amd._lib import PATH_MFMA_FUSED
+    if min(hw) < ks:
+        pytest.skip("image smaller than the window")
+    shape = (2, 3, hw[0], hw[1], D)
+    prev = _lib.enatten_set_path(PATH_MFMA_FUSED)
+    try:
+        q, k, v, g = make_inputs(shape, BF, seed=5)
+        print("case one-pass", shape, "k=%d" % ks, flush=True)
+        o, lse, dq, dk, dv = run_capi(q, k, v, g, ks)
+        ref = oracle_all(q, k, v, g, ks)
+        assert_close((o, dq, dk, dv), (ref[0], ref[2], ref[3], ref[4]), BF, "one-pass %s k%d" % (shape, ks))
+    finally:
+        _lib.enatten_set_path(prev)
+
+
+def test_one_pass_backward_fp16_and_strided_inputs(_lib):
+    # fp16, and q / k / v / dO read through the strides of a fused projection
+    from e_natten_amd import natten2d
+    from e_natten_amd._lib import PATH_MFMA_FUSED
+    prev = _lib.enatten_set_path(PATH_MFMA_FUSED)
+    try:
+        _case((1, 2, 30, 19, 32), F16, 7, seed=3, what="one-pass fp16")
+        B, N, H, W, D = 2, 4, 24, 20, 32
+        gen = torch.Generator().manual_seed(12)
+        qkv = torch.randn((B, H, W, 3, N, D), generator=gen).to(BF)
+        g = torch.randn((B, H, W, N, D), generator=gen).to(BF)
+        q, k, v = (qkv[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+        ref = oracle_all(q.contiguous(), k.contiguous(), v.contiguous(), g.permute(0, 3, 1, 2, 4).contiguous(), 5)
+        qkv_g = qkv.cuda().requires_grad_(True)
+        qg, kg, vg = (qkv_g[:, :, :, i].permute(0, 3, 1, 2, 4) for i in range(3))
+        o = natten2d(qg, kg, vg, 5)
+        (d_qkv,) = torch.autograd.grad(o, qkv_g, g.cuda().permute(0, 3, 1, 2, 4))
+        got = (o.detach().cpu(),) + tuple(d_qkv[:, :, :, i].permute(0, 3, 1, 2, 4).cpu() for i in range(3))
+        assert_close(got, (ref[0], ref[2], ref[3], ref[4]), BF, "one-pass strided")
+    finally:
+        _lib.enatten_set_path(prev)
+
+
 def test_config4_large_window(path):
     _case((2, 8, 128, 128, 64), BF, 13, what="C4")
 

@@ -63,6 +63,9 @@ def test_kernel_path_query(lib):
     from e_natten_amd import kernel_path
     assert kernel_path(128, 5, torch.float32) == "mfma"    # float32 matrix-core kernels
     assert kernel_path(128, 9, torch.float32) == "simt"
+    # every kernel size of the matrix-core kernels at head_dim 128, the largest windows included
+    assert all(kernel_path(128, ks, torch.bfloat16) == "mfma" for ks in (3, 5, 7, 9, 11, 13))
+    assert kernel_path(128, 13, torch.float16) == "mfma" and kernel_path(128, 15, torch.bfloat16) == "simt"
     assert kernel_path(2, 3, torch.float32) == "simt"
     assert kernel_path(128, 4, torch.bfloat16) == "none"
     assert kernel_path(4096, 3, torch.bfloat16) == "none"
