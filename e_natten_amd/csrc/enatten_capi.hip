@@ -23,6 +23,7 @@ namespace {
 
 int elem_size(int dtype) {
     switch (dtype) {
+        case ENATTEN_F64: return 8;
         case ENATTEN_F32: return 4;
         case ENATTEN_BF16:
         case ENATTEN_F16: return 2;
@@ -32,7 +33,7 @@ int elem_size(int dtype) {
 
 int check_shape(const char *fn, int B, int N, int H, int W, int D, int ks, int dtype) {
     if (elem_size(dtype) == 0) {
-        set_error("%s: unknown dtype code %d (expected ENATTEN_F32/BF16/F16)", fn, dtype);
+        set_error("%s: unknown dtype code %d (expected ENATTEN_F32/BF16/F16/F64)", fn, dtype);
         return ENATTEN_EINVAL;
     }
     if (B < 1 || N < 1 || H < 1 || W < 1 || D < 1) {
@@ -90,9 +91,19 @@ bool use_mfma_f32(int D, int ks, int dtype) {
     return g_path.load() != ENATTEN_PATH_SIMT && mfma_f32_supported(D, ks, dtype);
 }
 // float32 per query of backward workspace: two for the general and the 16-bit kernels
-// (delta and 1/Z), 2 * ks * ks for the float32 matrix-core kernels (P and dS)
+// (delta and 1/Z), 2 * ks * ks for the float32 matrix-core kernels (P and dS), four for
+// float64 tensors (two doubles: the log-sum-exp in double and delta)
 size_t ws_floats_per_query(int D, int ks, int dtype) {
+    if (dtype == ENATTEN_F64) return 4;
     return mfma_f32_supported(D, ks, dtype) ? mfma_f32_workspace_floats(ks) : 2;
+}
+// float64 tensors: one kernel family (na2d_f64.hip), whatever the path setting
+int bwd_f64(const char *fn, const BwdArgs &a, size_t ws_floats, hipStream_t st) {
+    if (ws_floats < (size_t)4 * a.s.B * a.s.N * a.s.H * a.s.W) {
+        set_error("%s: float64 tensors need 16 bytes of workspace per query", fn);
+        return ENATTEN_EUNSUPPORTED;
+    }
+    return launch_bwd_f64(a, st);
 }
 
 }  // namespace
@@ -136,6 +147,7 @@ int enatten2d_fwd(const void *q, const void *k, const void *v, void *o, float *l
     a.lse = lse;
     a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == ENATTEN_F64) return launch_fwd_f64(a, st);
     if (use_mfma(D, kernel_size, dtype)) return launch_fwd_mfma(a, dtype, st);
     if (use_mfma_f32(D, kernel_size, dtype)) return launch_fwd_mfma_f32(a, st);
     return launch_fwd_simt(a, dtype, st);
@@ -171,6 +183,7 @@ static int bwd2d(const char *fn, const void *q, const void *k, const void *v, co
     a.zinv = a.delta + (size_t)B * heads * H * W;
     a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == ENATTEN_F64) return bwd_f64(fn, a, ws_floats, st);
     if (use_mfma(D, kernel_size, dtype)) return launch_bwd_mfma(a, dtype, g_path.load(), st);
     // the float32 matrix-core backward where the workspace at hand holds its P and dS
     if (use_mfma_f32(D, kernel_size, dtype) &&
@@ -297,12 +310,13 @@ int enatten2d_fwd_window(const void *q, const void *k, const void *v, const void
     a.lse = lse;
     a.s = Shape{B, heads, H, W, D, kernel_h, kernel_w, scale, causal_h ? 1 : 0, causal_w ? 1 : 0};
     a.rpb = rpb;
+    if (dtype == ENATTEN_F64) return launch_fwd_f64(a, static_cast<hipStream_t>(stream));
     return launch_fwd_simt(a, dtype, static_cast<hipStream_t>(stream));
 }
 
 size_t enatten2d_bwd_window_workspace_bytes(int B, int heads, int H, int W) {
     if (B < 1 || heads < 1 || H < 1 || W < 1) return 0;
-    return (size_t)B * heads * H * W * 2 * sizeof(float);
+    return (size_t)B * heads * H * W * 4 * sizeof(float);  // float64 tensors use all four
 }
 
 int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void *rpb,
@@ -320,7 +334,7 @@ int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void
         set_error("%s: workspace is NULL", fn);
         return ENATTEN_EINVAL;
     }
-    const size_t ws_floats = (size_t)B * heads * H * W * 2;
+    const size_t ws_floats = (size_t)B * heads * H * W * (dtype == ENATTEN_F64 ? 4 : 2);
     if (plain)  // the reference's window: every kernel family that two floats per query allow
         return bwd2d(fn, q, k, v, o, d_o, lse, dq, dk, dv, static_cast<float *>(workspace),
                      ws_floats, B, heads, H, W, D, kernel_h, dtype, q_strides, k_strides, v_strides,
@@ -352,6 +366,7 @@ int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void
     a.s = Shape{B, heads, H, W, D, kernel_h, kernel_w, scale, causal_h ? 1 : 0, causal_w ? 1 : 0};
     a.rpb = rpb;
     a.d_rpb = d_rpb;
+    if (dtype == ENATTEN_F64) return bwd_f64(fn, a, ws_floats, static_cast<hipStream_t>(stream));
     return launch_bwd_simt(a, dtype, static_cast<hipStream_t>(stream));
 }
 
@@ -402,6 +417,7 @@ int enatten1d_fwd(const void *q, const void *k, const void *v, void *o, float *l
     if ((rc = view_1d(fn, "o", o, o_strides, heads, T, D, &a.o))) return rc;
     a.lse = lse;
     a.s = Shape{B, heads, 1, T, D, 1, kernel_size, scale};  // a 1 x k window on a 1 x T image
+    if (dtype == ENATTEN_F64) return launch_fwd_f64(a, static_cast<hipStream_t>(stream));
     if (g_path.load() != ENATTEN_PATH_SIMT && mfma1d_supported(D, kernel_size, dtype))
         return launch_fwd1d_mfma(a, dtype, static_cast<hipStream_t>(stream));
     return launch_fwd_simt(a, dtype, static_cast<hipStream_t>(stream));
@@ -409,7 +425,7 @@ int enatten1d_fwd(const void *q, const void *k, const void *v, void *o, float *l
 
 size_t enatten1d_bwd_workspace_bytes(int B, int heads, int T) {
     if (B < 1 || heads < 1 || T < 1) return 0;
-    return (size_t)B * heads * T * 2 * sizeof(float);
+    return (size_t)B * heads * T * 4 * sizeof(float);  // float64 tensors use all four
 }
 
 int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,
@@ -435,6 +451,8 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, co
     a.delta = static_cast<float *>(workspace);
     a.zinv = a.delta + (size_t)B * heads * T;
     a.s = Shape{B, heads, 1, T, D, 1, kernel_size, scale};
+    if (dtype == ENATTEN_F64)
+        return bwd_f64(fn, a, (size_t)4 * B * heads * T, static_cast<hipStream_t>(stream));
     if (g_path.load() != ENATTEN_PATH_SIMT && mfma1d_supported(D, kernel_size, dtype))
         return launch_bwd1d_mfma(a, dtype, g_path.load(), static_cast<hipStream_t>(stream));
     return launch_bwd_simt(a, dtype, static_cast<hipStream_t>(stream));

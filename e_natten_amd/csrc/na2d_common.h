@@ -100,6 +100,11 @@ struct ProfScope {
 int launch_fwd_simt(const FwdArgs &a, int dtype, hipStream_t st);
 int launch_bwd_simt(const BwdArgs &a, int dtype, hipStream_t st);
 
+// float64 tensors (plain double arithmetic; windows as the general kernels, no bias).  The
+// backward keeps two doubles per query in a.delta (16-byte aligned).
+int launch_fwd_f64(const FwdArgs &a, hipStream_t st);
+int launch_bwd_f64(const BwdArgs &a, hipStream_t st);
+
 // float32 matrix-core kernels (float64 logits): D in {32, 64, 128}, kernel_size 3 / 5 / 7.
 // Their backward keeps 2 * ks * ks float32 per query in the workspace (a.delta).
 bool mfma_f32_supported(int D, int ks, int dtype);

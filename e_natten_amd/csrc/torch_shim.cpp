@@ -30,6 +30,7 @@ int dtype_code(const Tensor &t) {
         case at::kFloat: return ENATTEN_F32;
         case at::kBFloat16: return ENATTEN_BF16;
         case at::kHalf: return ENATTEN_F16;
+        case at::kDouble: return ENATTEN_F64;
         default: return -1;
     }
 }
@@ -48,7 +49,7 @@ void validate(const char *what, const Tensor &q, const Tensor &k, const Tensor &
     TORCH_CHECK_VALUE(k.scalar_type() == q.scalar_type() && v.scalar_type() == q.scalar_type(),
                       what, ": q, k and v must share a dtype");
     TORCH_CHECK_VALUE(dtype_code(q) >= 0, what, ": dtype ", q.scalar_type(),
-                      " is not supported (float32, bfloat16, float16)");
+                      " is not supported (float32, bfloat16, float16, float64)");
     TORCH_CHECK_VALUE(k.device() == q.device() && v.device() == q.device(), what,
                       ": q, k and v must be on the same device");
     TORCH_CHECK_VALUE(ks >= 1 && ks % 2 == 1, what, ": kernel_size must be odd and >= 1, got ", ks);

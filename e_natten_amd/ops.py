@@ -24,7 +24,8 @@ import torch
 
 from . import _lib
 
-_DTYPES = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
+_DTYPES = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16,
+           torch.float64: _lib.F64}
 
 
 def _validate(q, k, v, kernel_size: int, ndim: int = 5) -> None:
@@ -41,7 +42,7 @@ def _validate(q, k, v, kernel_size: int, ndim: int = 5) -> None:
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise ValueError("q, k and v must share a dtype")
     if q.dtype not in _DTYPES:
-        raise ValueError("dtype %s is not supported (float32, bfloat16, float16)" % q.dtype)
+        raise ValueError("dtype %s is not supported (float32, bfloat16, float16, float64)" % q.dtype)
     if k.device != q.device or v.device != q.device:
         raise ValueError("q, k and v must be on the same device")
     if not isinstance(kernel_size, int) or isinstance(kernel_size, bool):

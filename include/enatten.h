@@ -26,10 +26,12 @@
 extern "C" {
 #endif
 
-#define ENATTEN_ABI_VERSION 4
+#define ENATTEN_ABI_VERSION 5
 
-/* element types of q, k, v, o and the gradients */
-enum { ENATTEN_F32 = 0, ENATTEN_BF16 = 1, ENATTEN_F16 = 2 };
+/* element types of q, k, v, o and the gradients.  ENATTEN_F64 runs in plain double
+ * arithmetic on kernels of its own (for numerical gradient checks, as the reference's
+ * gradcheck.py:6-15 does; not tuned); lse stays float32. */
+enum { ENATTEN_F32 = 0, ENATTEN_BF16 = 1, ENATTEN_F16 = 2, ENATTEN_F64 = 3 };
 
 /* return codes */
 enum {
@@ -91,7 +93,8 @@ int enatten2d_fwd(const void *q, const void *k, const void *v, void *o, float *l
  * Bytes of device scratch enatten2d_bwd needs for a call of this shape: two float32
  * per query, or 2 * kernel_size^2 per query where the float32 matrix-core kernels
  * serve the call (they hand the probabilities and their gradients from the dQ pass to
- * the dK/dV pass through it).
+ * the dK/dV pass through it), or two doubles per query for float64 tensors (16-byte
+ * aligned).
  */
 size_t enatten2d_bwd_workspace_bytes(int B, int heads, int H, int W, int D, int kernel_size,
                                      int dtype);
@@ -155,8 +158,8 @@ int enatten2d_bwd_static(const void *q, const void *k, const void *v, const void
  * k positions up to and including its own, fewer at the start of the axis, and k may be
  * even there; on the other axes the window is the reference's
  * clamp(i - k/2, 0, L - k) with k odd.  The same conventions as enatten2d_fwd /
- * enatten2d_bwd otherwise; the workspace holds two float32 per query
- * (enatten2d_bwd_window_workspace_bytes).  A 1D causal (sliding-window) attention over
+ * enatten2d_bwd otherwise; the workspace holds 16 bytes per query
+ * (enatten2d_bwd_window_workspace_bytes: two float32, or two doubles for float64 tensors).  A 1D causal (sliding-window) attention over
  * [B, heads, T, D] is the call with H = 1, kernel_h = 1, causal_h = 0.
  *
  * rpb, NULL or a relative position bias [heads, 2 * kernel_h - 1, 2 * kernel_w - 1] of the
@@ -197,6 +200,7 @@ int enatten1d_fwd(const void *q, const void *k, const void *v, void *o, float *l
                   const int64_t *q_strides, const int64_t *k_strides,
                   const int64_t *v_strides, const int64_t *o_strides, float scale,
                   void *stream);
+/* 16 bytes per position: two float32, or two doubles for float64 tensors (16-byte aligned) */
 size_t enatten1d_bwd_workspace_bytes(int B, int heads, int T);
 int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o,
                   const void *d_o, const float *lse, void *dq, void *dk, void *dv,

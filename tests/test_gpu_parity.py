@@ -725,3 +725,39 @@ def test_relative_position_bias(shape, kernel, dtype, dil, _lib):
            else O.rel_err(d_rpb, d_ref))
     print("   d_rpb err %.3e" % err, flush=True)
     assert err <= (1e-4 if dtype == F32 else BF16_REL)
+
+
+@pytest.mark.parametrize("shape,ks", [((2, 3, 8, 2), 7), ((1, 2, 11, 5), 3)])
+def test_float64_gradcheck_1d(shape, ks, _lib):
+    # the reference's own gradient check (gradcheck.py:6-15: float64 (2, 3, 8, 2), kernel_size 7,
+    # eps 1e-6, atol 1e-4), run on this operator itself
+    from e_natten_amd import natten1d
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(shape, generator=g, dtype=torch.float64).cuda().requires_grad_(True) for _ in range(3))
+    print("case float64 gradcheck 1d", shape, ks, flush=True)
+    assert torch.autograd.gradcheck(lambda a, b, c: natten1d(a, b, c, ks), (q, k, v), eps=1e-6, atol=1e-4)
+
+
+@pytest.mark.parametrize("shape,ks", [((1, 2, 6, 7, 3), 3), ((2, 1, 5, 5, 2), 5), ((1, 1, 9, 8, 4), 7)])
+def test_float64_gradcheck_2d(shape, ks, _lib):
+    from e_natten_amd import natten2d
+    g = torch.Generator().manual_seed(1)
+    q, k, v = (torch.randn(shape, generator=g, dtype=torch.float64).cuda().requires_grad_(True) for _ in range(3))
+    print("case float64 gradcheck 2d", shape, ks, flush=True)
+    assert torch.autograd.gradcheck(lambda a, b, c: natten2d(a, b, c, ks, 0.7), (q, k, v), eps=1e-6, atol=1e-4)
+
+
+@pytest.mark.parametrize("shape,ks", [((2, 2, 16, 13, 24), 5), ((1, 2, 20, 20, 130), 3), ((1, 1, 9, 9, 8), 9)])
+def test_float64_against_the_oracle(shape, ks, _lib):
+    # float64 tensors in plain double arithmetic: agreement with the float64 oracle to 1e-10
+    from e_natten_amd import natten2d
+    g = torch.Generator().manual_seed(2)
+    q, k, v, d_o = (torch.randn(shape, generator=g, dtype=torch.float64) for _ in range(4))
+    ref = O.natten2d_explicit(q, k, v, d_o, ks, 1.0, compute_dtype=torch.float64)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = natten2d(qg, kg, vg, ks)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), d_o.cuda())
+    for name, x, r in zip(("O", "dQ", "dK", "dV"), (o, dq, dk, dv), (ref[0], ref[2], ref[3], ref[4])):
+        err = (x.detach().cpu() - r.double()).abs().max().item()
+        print("   float64", name, "max-abs err %.2e" % err, flush=True)
+        assert err <= 1e-10 * max(1.0, r.abs().max().item()), (name, err)

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol(lib):
     for n in names:
         assert hasattr(lib, n), "libenatten.so does not export %s" % n
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.enatten_abi_version() == _lib.ABI_VERSION == 4
+    assert lib.enatten_abi_version() == _lib.ABI_VERSION == 5
 
 
 def test_c_abi_validates_before_launch(lib):
@@ -69,7 +69,8 @@ def test_kernel_path_query(lib):
     assert kernel_path(2, 3, torch.float32) == "simt"
     assert kernel_path(128, 4, torch.bfloat16) == "none"
     assert kernel_path(4096, 3, torch.bfloat16) == "none"
-    assert kernel_path(128, 5, torch.float64) == "none"
+    assert kernel_path(128, 5, torch.float64) == "simt"    # float64: kernels of their own, not matrix-core
+    assert kernel_path(128, 5, torch.int32) == "none"
     prev = lib.enatten_set_path(1)
     assert kernel_path(128, 5, torch.bfloat16) == "simt"
     lib.enatten_set_path(prev)
@@ -90,7 +91,7 @@ def test_native_torch_binding_registers_operators():
     with pytest.raises(ValueError, match="same shape"):
         torch.ops.enatten.na2d_fwd(q, q[:, :, :4], q, 3, 1.0)
     with pytest.raises(ValueError, match="dtype"):
-        torch.ops.enatten.natten2d(q.double(), q.double(), q.double(), 3, 1.0)
+        torch.ops.enatten.natten2d(q.int(), q.int(), q.int(), 3, 1.0)
     with pytest.raises(RuntimeError, match="no CPU path"):
         torch.ops.enatten.natten2d(q, q, q, 3, 1.0)
     with pytest.raises(RuntimeError, match="no CPU path"):
@@ -146,7 +147,7 @@ def test_1d_surface_and_validation(lib):
                                           None, None, 1.0, None)
     assert f(4) == 1 and "odd" in _lib.last_error()
     assert f(9) == 1 and "smaller" in _lib.last_error()
-    assert lib.enatten1d_bwd_workspace_bytes(2, 3, 10) == 2 * 3 * 10 * 8
+    assert lib.enatten1d_bwd_workspace_bytes(2, 3, 10) == 2 * 3 * 10 * 16  # two doubles per position for float64 tensors
     # The size limit is on B * heads * T * D elements, not on a T x T image: long
     # sequences pass it and fail on the NULL pointer that follows (nothing is launched).
     for B, N, T, D in ((8, 8, 16384, 128), (1, 8, 131072, 64), (1, 1, 1 << 22, 64)):
@@ -168,7 +169,7 @@ def test_python_validation_without_gpu():
     with pytest.raises(ValueError):
         natten2d(q, q[:, :, :4], q, 3)
     with pytest.raises(ValueError):
-        natten2d(q.double(), q.double(), q.double(), 3)
+        natten2d(q.int(), q.int(), q.int(), 3)
     with pytest.raises(TypeError):
         natten2d(q, q, q, 3.0)
     # valid arguments on CPU tensors: there is no CPU path, so this must fail loudly
@@ -213,7 +214,7 @@ def test_window_entry_points_validate(lib):
     assert f(3, 0, 0, 1) == 1
     assert f(3, 4, 0, 1, q=None) == 1 and "q is NULL" in _lib.last_error()   # even is fine when causal
     assert f(4, 4) == 1 and "odd" in _lib.last_error()   # square non-causal: the plain entry point's rule
-    assert lib.enatten2d_bwd_window_workspace_bytes(2, 3, 4, 5) == 2 * 3 * 4 * 5 * 8
+    assert lib.enatten2d_bwd_window_workspace_bytes(2, 3, 4, 5) == 2 * 3 * 4 * 5 * 16
     assert f(3, 5, 0, 1, rpb=1) == 1 and "centred axes only" in _lib.last_error()
     assert lib.enatten2d_bwd_window(1, 1, 1, None, 1, 1, None, 1, 1, 1, None, None, 1, 1, 8, 8, 16, 3, 5,
                                     0, 0, 0, None, None, None, None, None, 1.0, None) == 1
