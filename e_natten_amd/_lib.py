@@ -29,13 +29,15 @@ SIGNATURES = {
     "enatten2d_fwd": (_i, [_vp] * 5 + [_i] * 7 + [_sp] * 4 + [ctypes.c_float, _vp]),
     "enatten2d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 7),
     "enatten2d_bwd": (_i, [_vp] * 10 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
+    "enatten2d_bwd_into": (_i, [_vp] * 10 + [_i] * 7 + [_sp] * 6 + [ctypes.c_float, _vp]),
     "enatten2d_bwd_static": (_i, [_vp] * 9 + [_i] * 7 + [_sp] * 5 + [ctypes.c_float, _vp]),
     "enatten2d_fwd_window": (_i, [_vp] * 6 + [_i] * 10 + [_sp] * 4 + [ctypes.c_float, _vp]),
-    "enatten2d_bwd_window_workspace_bytes": (ctypes.c_size_t, [_i] * 4),
+    "enatten2d_bwd_window_workspace_bytes": (ctypes.c_size_t, [_i] * 7),
     "enatten2d_bwd_window": (_i, [_vp] * 12 + [_i] * 10 + [_sp] * 5 + [ctypes.c_float, _vp]),
     "enatten1d_fwd": (_i, [_vp] * 5 + [_i] * 6 + [_sp] * 4 + [ctypes.c_float, _vp]),
     "enatten1d_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 3),
     "enatten1d_bwd": (_i, [_vp] * 10 + [_i] * 6 + [_sp] * 5 + [ctypes.c_float, _vp]),
+    "enatten1d_bwd_into": (_i, [_vp] * 10 + [_i] * 6 + [_sp] * 6 + [ctypes.c_float, _vp]),
     "enatten_profile_enable": (_i, [_i]),
     "enatten_profile_read": (_i, [_i, ctypes.POINTER(_i), ctypes.POINTER(ctypes.c_double)]),
     "enatten_profile_kernel_name": (ctypes.c_char_p, [_i]),

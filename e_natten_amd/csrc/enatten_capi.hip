@@ -97,6 +97,24 @@ size_t ws_floats_per_query(int D, int ks, int dtype) {
     if (dtype == ENATTEN_F64) return 4;
     return mfma_f32_supported(D, ks, dtype) ? mfma_f32_workspace_floats(ks) : 2;
 }
+// Layout of dq, dk, dv: contiguous [B, heads, H, W, D], or the caller's element strides on
+// (batch, head, row, column) with unit stride on the channels.  Call after a->s is set.
+int set_grad_layout(const char *fn, BwdArgs *a, const int64_t *st) {
+    const Shape &s = a->s;
+    if (st) {
+        a->gsb = st[0]; a->gsn = st[1]; a->gsh = st[2]; a->gsw = st[3];
+        if (a->gsb < 0 || a->gsn < 0 || a->gsh < 0 || a->gsw < s.D) {
+            set_error("%s: gradient strides must be non-negative, and at least D between pixels", fn);
+            return ENATTEN_EINVAL;
+        }
+    } else {
+        a->gsw = s.D;
+        a->gsh = (int64_t)s.W * s.D;
+        a->gsn = (int64_t)s.H * s.W * s.D;
+        a->gsb = (int64_t)s.N * s.H * s.W * s.D;
+    }
+    return ENATTEN_OK;
+}
 // float64 tensors: one kernel family (na2d_f64.hip), whatever the path setting
 int bwd_f64(const char *fn, const BwdArgs &a, size_t ws_floats, hipStream_t st) {
     if (ws_floats < (size_t)4 * a.s.B * a.s.N * a.s.H * a.s.W) {
@@ -165,7 +183,7 @@ static int bwd2d(const char *fn, const void *q, const void *k, const void *v, co
                  float *workspace, size_t ws_floats, int B, int heads, int H, int W, int D, int kernel_size,
                  int dtype, const int64_t *q_strides, const int64_t *k_strides,
                  const int64_t *v_strides, const int64_t *o_strides, const int64_t *do_strides,
-                 float scale, void *stream) {
+                 float scale, void *stream, const int64_t *grad_strides = nullptr) {
     BwdArgs a;
     int rc;
     if ((rc = make_view(fn, "q", q, q_strides, heads, H, W, D, &a.q))) return rc;
@@ -182,11 +200,13 @@ static int bwd2d(const char *fn, const void *q, const void *k, const void *v, co
     a.delta = workspace;
     a.zinv = a.delta + (size_t)B * heads * H * W;
     a.s = Shape{B, heads, H, W, D, kernel_size, kernel_size, scale};
+    if ((rc = set_grad_layout(fn, &a, grad_strides))) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (dtype == ENATTEN_F64) return bwd_f64(fn, a, ws_floats, st);
     if (use_mfma(D, kernel_size, dtype)) return launch_bwd_mfma(a, dtype, g_path.load(), st);
-    // the float32 matrix-core backward where the workspace at hand holds its P and dS
-    if (use_mfma_f32(D, kernel_size, dtype) &&
+    // the float32 matrix-core backward where the workspace at hand holds its P and dS (it
+    // writes contiguous gradients only)
+    if (use_mfma_f32(D, kernel_size, dtype) && a.grads_contiguous() &&
         ws_floats >= (size_t)B * heads * H * W * mfma_f32_workspace_floats(kernel_size))
         return launch_bwd_mfma_f32(a, st);
     return launch_bwd_simt(a, dtype, st);
@@ -210,6 +230,26 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o, co
                  (size_t)B * heads * H * W * ws_floats_per_query(D, kernel_size, dtype), B, heads,
                  H, W, D, kernel_size, dtype, q_strides, k_strides, v_strides, o_strides,
                  do_strides, scale, stream);
+}
+
+int enatten2d_bwd_into(const void *q, const void *k, const void *v, const void *o,
+                       const void *d_o, const float *lse, void *dq, void *dk, void *dv,
+                       void *workspace, int B, int heads, int H, int W, int D, int kernel_size,
+                       int dtype, const int64_t *q_strides, const int64_t *k_strides,
+                       const int64_t *v_strides, const int64_t *o_strides,
+                       const int64_t *do_strides, const int64_t *grad_strides, float scale,
+                       void *stream) {
+    const char *fn = "enatten2d_bwd_into";
+    const int rc = check_shape(fn, B, heads, H, W, D, kernel_size, dtype);
+    if (rc) return rc;
+    if (!workspace) {
+        set_error("%s: workspace is NULL", fn);
+        return ENATTEN_EINVAL;
+    }
+    return bwd2d(fn, q, k, v, o, d_o, lse, dq, dk, dv, static_cast<float *>(workspace),
+                 (size_t)B * heads * H * W * ws_floats_per_query(D, kernel_size, dtype), B, heads,
+                 H, W, D, kernel_size, dtype, q_strides, k_strides, v_strides, o_strides,
+                 do_strides, scale, stream, grad_strides);
 }
 
 // ---- backward without a caller-provided workspace ---------------------------
@@ -314,9 +354,12 @@ int enatten2d_fwd_window(const void *q, const void *k, const void *v, const void
     return launch_fwd_simt(a, dtype, static_cast<hipStream_t>(stream));
 }
 
-size_t enatten2d_bwd_window_workspace_bytes(int B, int heads, int H, int W) {
-    if (B < 1 || heads < 1 || H < 1 || W < 1) return 0;
-    return (size_t)B * heads * H * W * 4 * sizeof(float);  // float64 tensors use all four
+size_t enatten2d_bwd_window_workspace_bytes(int B, int heads, int H, int W, int kernel_h,
+                                            int kernel_w, int with_rpb) {
+    if (B < 1 || heads < 1 || H < 1 || W < 1 || kernel_h < 1 || kernel_w < 1) return 0;
+    // four floats per query (float64 tensors use all four), and with a bias dS of every
+    // (query, window position)
+    return (size_t)B * heads * H * W * (4 + (with_rpb ? (size_t)kernel_h * kernel_w : 0)) * sizeof(float);
 }
 
 int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void *rpb,
@@ -364,8 +407,10 @@ int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void
     a.delta = static_cast<float *>(workspace);
     a.zinv = a.delta + (size_t)B * heads * H * W;
     a.s = Shape{B, heads, H, W, D, kernel_h, kernel_w, scale, causal_h ? 1 : 0, causal_w ? 1 : 0};
+    if ((rc = set_grad_layout(fn, &a, nullptr))) return rc;
     a.rpb = rpb;
     a.d_rpb = d_rpb;
+    a.ds_pairs = rpb ? a.delta + (size_t)4 * B * heads * H * W : nullptr;
     if (dtype == ENATTEN_F64) return bwd_f64(fn, a, ws_floats, static_cast<hipStream_t>(stream));
     return launch_bwd_simt(a, dtype, static_cast<hipStream_t>(stream));
 }
@@ -433,7 +478,18 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, co
                   int heads, int T, int D, int kernel_size, int dtype, const int64_t *q_strides,
                   const int64_t *k_strides, const int64_t *v_strides, const int64_t *o_strides,
                   const int64_t *do_strides, float scale, void *stream) {
-    const char *fn = "enatten1d_bwd";
+    return enatten1d_bwd_into(q, k, v, o, d_o, lse, dq, dk, dv, workspace, B, heads, T, D, kernel_size,
+                              dtype, q_strides, k_strides, v_strides, o_strides, do_strides, nullptr,
+                              scale, stream);
+}
+
+int enatten1d_bwd_into(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                       const float *lse, void *dq, void *dk, void *dv, void *workspace, int B,
+                       int heads, int T, int D, int kernel_size, int dtype,
+                       const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                       const int64_t *o_strides, const int64_t *do_strides,
+                       const int64_t *grad_strides, float scale, void *stream) {
+    const char *fn = grad_strides ? "enatten1d_bwd_into" : "enatten1d_bwd";
     int rc = check_shape_1d(fn, B, heads, T, D, kernel_size, dtype);
     if (rc) return rc;
     BwdArgs a;
@@ -451,6 +507,12 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o, co
     a.delta = static_cast<float *>(workspace);
     a.zinv = a.delta + (size_t)B * heads * T;
     a.s = Shape{B, heads, 1, T, D, 1, kernel_size, scale};
+    {
+        // (batch, head, position) strides -> the four of an image with one row
+        const int64_t g4[4] = {grad_strides ? grad_strides[0] : 0, grad_strides ? grad_strides[1] : 0, 0,
+                               grad_strides ? grad_strides[2] : 0};
+        if ((rc = set_grad_layout(fn, &a, grad_strides ? g4 : nullptr))) return rc;
+    }
     if (dtype == ENATTEN_F64)
         return bwd_f64(fn, a, (size_t)4 * B * heads * T, static_cast<hipStream_t>(stream));
     if (g_path.load() != ENATTEN_PATH_SIMT && mfma1d_supported(D, kernel_size, dtype))

@@ -318,7 +318,7 @@ __global__ __launch_bounds__(256, 2) void bwd1d_dq_mfma(BwdArgs a, int tiles_t, 
                     dq[mt] = mfma16<BF>(cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)),
                                         dsb[kk], dq[mt]);
             }
-            store_token<BF, D>(static_cast<short *>(a.dq) + lq.tok * D, g, dq, s.scale, lq.live);
+            store_token<BF, D>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, 0, lq.qt), g, dq, s.scale, lq.live);
             if (lq.live && g == 0) a.delta[lq.tok] = delta;
         }
         if (!more) break;
@@ -444,10 +444,10 @@ __global__ __launch_bounds__(256, 2) void bwd1d_dkdv_mfma(BwdArgs a, int tiles_t
                     dk[mt] = mfma16<BF>(cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)), dsb, dk[mt]);
                 }
             }
-            const int64_t tok = ((int64_t)cur.bb * s.N + cur.nn) * T + kt;
+            const int64_t goff = a.grad_at(cur.bb, cur.nn, 0, kt);
             const bool live = w0 + n < T;
-            store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, live);
-            store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, live);
+            store_token<BF, D>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live);
+            store_token<BF, D>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live);
         }
         if (!more) break;
         load_keys(nxt);
@@ -536,7 +536,7 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
         if (w0 < T) {
             const bool live = w0 + n < T;
             const int pt = min(w0 + n, T - 1);  // this lane's position, as query and as key
-            const int64_t tok = ((int64_t)cur.bb * s.N + cur.nn) * T + pt;
+            const int64_t goff = a.grad_at(cur.bb, cur.nn, 0, pt);
             const int own = pt - ra;
             {
                 // ---- dQ: the wave's keys are the 16 + k - 1 positions from the window start
@@ -586,7 +586,7 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
                         dq[mt] = mfma16<BF>(cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)),
                                             dsb[kk], dq[mt]);
                 }
-                store_token<BF, D>(static_cast<short *>(a.dq) + tok * D, g, dq, s.scale, live);
+                store_token<BF, D>(static_cast<short *>(a.dq) + goff, g, dq, s.scale, live);
             }
             {
                 // ---- dK, dV: the queries that attend to any of the wave's 16 keys, 32 at a time
@@ -643,8 +643,8 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
                         dk[mt] = mfma16<BF>(cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)), dsb, dk[mt]);
                     }
                 }
-                store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, live);
-                store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, live);
+                store_token<BF, D>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live);
+                store_token<BF, D>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live);
             }
         }
         if (!more) break;
@@ -746,7 +746,7 @@ bool fused1d_supported(const BwdArgs &a) {
 int launch_bwd1d_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st) {
     auto al = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
     if (!layout1d_ok(a.q) || !layout1d_ok(a.k) || !layout1d_ok(a.v) || !layout1d_ok(a.d_o) ||
-        !al(a.dq) || !al(a.dk) || !al(a.dv))
+        !al(a.dq) || !al(a.dk) || !al(a.dv) || a.gsb % 8 != 0 || a.gsn % 8 != 0 || a.gsw % 8 != 0)
         return launch_bwd_simt(a, dtype, st);
     if (path != ENATTEN_PATH_MFMA_SPLIT && fused1d_supported(a)) {
         ENATTEN_1D(bwd1d_fused_launch, a, dtype, st)

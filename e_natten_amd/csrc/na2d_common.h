@@ -33,12 +33,25 @@ struct BwdArgs {
     View q, k, v;
     View o, d_o;  // forward output and upstream gradient, strided views like q, k, v
     const float *lse;
-    void *dq, *dk, *dv;  // contiguous
+    void *dq, *dk, *dv;
+    // element strides of dq, dk and dv alike on (batch, head, row, column), unit stride on the
+    // channels: contiguous tensors unless the caller writes the gradients into strided views
+    // (the sub-grids of a dilated call); set_grad_layout fills them
+    int64_t gsb, gsn, gsh, gsw;
+    __host__ __device__ int64_t grad_at(int b, int n, int y, int x) const {
+        return b * gsb + n * gsn + y * gsh + x * gsw;
+    }
+    bool grads_contiguous() const {
+        return gsw == s.D && gsh == (int64_t)s.W * s.D && gsn == (int64_t)s.H * s.W * s.D &&
+               gsb == (int64_t)s.N * s.H * s.W * s.D;
+    }
     float *delta;        // scratch [B, N, H, W]: sum_j P_j dP_j per query
     float *zinv;         // scratch [B, N, H, W]: 1 / sum_j exp(S_j - lse) (vector-ALU kernels)
     Shape s;
     const void *rpb = nullptr;  // relative position bias [N, 2*kh-1, 2*kw-1] in the tensors' type
-    float *d_rpb = nullptr;     // its gradient, float32, accumulated with atomics (general kernels)
+    float *d_rpb = nullptr;     // its gradient, float32, fully overwritten (general kernels)
+    float *ds_pairs = nullptr;  // scratch [B, N, H, W, kh*kw]: dS of every (query, window position),
+                                // from which d_rpb is summed in a fixed order
 };
 
 // NATTEN window start on an axis of length L: centred, shifted to stay inside

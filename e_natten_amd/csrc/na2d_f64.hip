@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256) void bwd_dq_f64(BwdArgs a, double2 *stat) {
                 if (lane + 64 * i < s.D) dq[i] = fma(ds, kp[lane + 64 * i], dq[i]);
         }
     if (!px.live) return;
-    double *out = static_cast<double *>(a.dq) + px.tok * s.D;
+    double *out = static_cast<double *>(a.dq) + a.grad_at(px.b, px.n, px.y, px.x);
 #pragma unroll
     for (int i = 0; i < NCH; i++)
         if (lane + 64 * i < s.D) out[lane + 64 * i] = dq[i] * (double)s.scale;
@@ -165,7 +165,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_f64(BwdArgs a, const double2 *st
                 }
         }
     if (!px.live) return;
-    double *okp = static_cast<double *>(a.dk) + px.tok * s.D, *ovp = static_cast<double *>(a.dv) + px.tok * s.D;
+    const int64_t goff = a.grad_at(px.b, px.n, px.y, px.x);
+    double *okp = static_cast<double *>(a.dk) + goff, *ovp = static_cast<double *>(a.dv) + goff;
 #pragma unroll
     for (int i = 0; i < NCH; i++)
         if (lane + 64 * i < s.D) {

@@ -464,7 +464,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void b
                         dq[mt]);
             }
 
-            store_token<BF, D>(static_cast<short *>(a.dq) + lq.tok * D, g, dq, s.scale, lq.live);
+            store_token<BF, D>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live);
             if (lq.live && g == 0) a.delta[lq.tok] = delta;
         }
 
@@ -599,7 +599,7 @@ __global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void bwd_dq2_mfma(BwdArg
                         cat(lds_read_tr(G::t_at(kp[0], mt)), lds_read_tr(G::t_at(kp[1], mt))), dsb[ks],
                         dq[mt]);
             }
-            store_token<BF, D>(static_cast<short *>(a.dq) + lq.tok * D, g, dq, s.scale, lq.live);
+            store_token<BF, D>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live);
             if (lq.live && g == 0) a.delta[lq.tok] = delta;
         }
         if (!more) break;
@@ -813,10 +813,10 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         }
 
         const int kr = cur.r0 + orow + (n >> 2), kc = cur.c0 + ocol + (n & 3);
-        const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + kr) * s.W + kc;
+        const int64_t goff = a.grad_at(cur.bb, cur.nn, kr, kc);
         if constexpr (SP == 1) {
-            store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
-            store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
+            store_token<BF, D>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, true);
+            store_token<BF, D>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, true);
             if (!more) break;
             load_keys(nxt);
             __syncthreads();
@@ -841,8 +841,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
                     dk[mt] += red[mt * 256];
                     dv[mt] += red[(G::DT + mt) * 256];
                 }
-                store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
-                store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
+                store_token<BF, D>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, true);
+                store_token<BF, D>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, true);
             }
             if (!more) break;
         }
@@ -1024,10 +1024,9 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 
         const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
         auto store = [&]() __attribute__((always_inline)) {
-            const int64_t tok =
-                (((int64_t)cur.tl.bb * s.N + cur.tl.nn) * s.H + kr) * s.W + kc;
-            store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, live);
-            store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, live);
+            const int64_t goff = a.grad_at(cur.tl.bb, cur.tl.nn, kr, kc);
+            store_token<BF, D>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live);
+            store_token<BF, D>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live);
         };
         if constexpr (SP == 1) {
             if (cur.last) store();
@@ -1383,8 +1382,9 @@ int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st) {
 
 int launch_bwd_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st) {
     auto al = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const bool grads_ok = a.gsb % 8 == 0 && a.gsn % 8 == 0 && a.gsh % 8 == 0 && a.gsw % 8 == 0;
     if (!layout_ok(a.q) || !layout_ok(a.k) || !layout_ok(a.v) || !layout_ok(a.o) ||
-        !layout_ok(a.d_o) || !al(a.dq) || !al(a.dk) || !al(a.dv))
+        !layout_ok(a.d_o) || !al(a.dq) || !al(a.dk) || !al(a.dv) || !grads_ok)
         return launch_bwd_simt(a, dtype, st);
     if (dtype == ENATTEN_BF16) {
         ENATTEN_BY_D(bwd_launch, true, a, path, st)

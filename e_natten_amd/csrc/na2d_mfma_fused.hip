@@ -735,6 +735,7 @@ bool fused_bwd_supported(const BwdArgs &a) {
         return ((int64_t)a.s.H * v.sh + (int64_t)a.s.W * v.sw + a.s.D) * 2 < ((int64_t)1 << 32);
     };
     return a.s.D == 128 && a.s.kh == 5 && a.s.kw == 5 && a.s.H % 8 == 0 && a.s.W % 8 == 0 &&
+           a.grads_contiguous() &&
            small(a.q) && small(a.k) && small(a.v) && small(a.o) && small(a.d_o);
 }
 

@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256, 2) void bwd_onepass_mfma(BwdArgs a, TileSet ts
         const int py = wy0 + (n >> 2), px = wx0 + (n & 3);
         const bool live = (cur.last_r || py < s.H - 8) && (cur.last_c || px < s.W - 8);
         const int prow = (py - br) * G::HC + (px - bc);
-        const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + py) * s.W + px;
+        const int64_t goff = a.grad_at(cur.bb, cur.nn, py, px);
         {
             // ---- dQ: the wave's keys are the (4+k-1)^2 pixels from the window start of its
             // first query row / column on (moved back where that would leave the block)
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256, 2) void bwd_onepass_mfma(BwdArgs a, TileSet ts
                         cat(lds_read_tr(G::t_at(kp[0], mt)), lds_read_tr(G::t_at(kp[1], mt))), dsb[ks],
                         dq[mt]);
             }
-            store_token<BF, D>(static_cast<short *>(a.dq) + tok * D, g, dq, s.scale, live);
+            store_token<BF, D>(static_cast<short *>(a.dq) + goff, g, dq, s.scale, live);
         }
         __builtin_amdgcn_sched_barrier(0);
         if (more) prefetch_vgo(nxt);
@@ -329,8 +329,8 @@ __global__ __launch_bounds__(256, 2) void bwd_onepass_mfma(BwdArgs a, TileSet ts
                     }
                 }
             }
-            store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, live);
-            store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, live);
+            store_token<BF, D>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live);
+            store_token<BF, D>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live);
         }
 
         if (!more) break;

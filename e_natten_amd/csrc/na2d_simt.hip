@@ -297,7 +297,7 @@ __global__ __launch_bounds__(256) void bwd_dq_simt(BwdArgs a, int tiles_x, int t
     if (!pl.live) return;
     const float zinv = 1.f / zsum;
     const float shift = esum * zinv;
-    T *dqp = static_cast<T *>(a.dq) + tok * s.D;
+    T *dqp = static_cast<T *>(a.dq) + a.grad_at(pl.b, pl.n, pl.x, pl.y);  // (pl.x is the row)
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         const int d0 = (c * G + pl.lg) * 8;
@@ -358,10 +358,12 @@ __global__ __launch_bounds__(256) void bwd_dkdv_simt(BwdArgs a, int tiles_x, int
             const float p = exp_neg(sl - (A)a.lse[qtok]) * a.zinv[qtok];
             const float ds = p * (group_sum<G>(pd) - a.delta[qtok]);
             // d(bias) of this (query, key) pair is dS itself; here P and dS are final (the
-            // dQ pass left 1 / Z and the corrected delta)
-            if (a.d_rpb && pl.live && pl.lg == 0)
-                atomicAdd(a.d_rpb + ((int64_t)pl.n * (2 * s.kh - 1) + (pl.x - xi + s.kh - 1)) *
-                                        (2 * s.kw - 1) + (pl.y - yi + s.kw - 1), ds);
+            // dQ pass left 1 / Z and the corrected delta).  It is left at the pair's place in
+            // the query's window (every place is written exactly once, by the one key it
+            // names), and rpb_grad_reduce sums the places of a bias entry in a fixed order.
+            if (a.ds_pairs && pl.live && pl.lg == 0)
+                a.ds_pairs[qtok * (s.kh * s.kw) + (pl.x - win_start(xi, s.H, s.kh)) * s.kw +
+                           (pl.y - win_start(yi, s.W, s.kw))] = ds;
 #pragma unroll
             for (int c = 0; c < CH; c++)
 #pragma unroll
@@ -372,9 +374,9 @@ __global__ __launch_bounds__(256) void bwd_dkdv_simt(BwdArgs a, int tiles_x, int
         }
     }
     if (!pl.live) return;
-    const int64_t tok = img + (int64_t)pl.x * s.W + pl.y;
-    T *dkp = static_cast<T *>(a.dk) + tok * s.D;
-    T *dvp = static_cast<T *>(a.dv) + tok * s.D;
+    const int64_t goff = a.grad_at(pl.b, pl.n, pl.x, pl.y);
+    T *dkp = static_cast<T *>(a.dk) + goff;
+    T *dvp = static_cast<T *>(a.dv) + goff;
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         const int d0 = (c * G + pl.lg) * 8;
@@ -383,6 +385,34 @@ __global__ __launch_bounds__(256) void bwd_dkdv_simt(BwdArgs a, int tiles_x, int
         store8<T, VEC>(dkp + d0, s.D - d0, dk[c]);
         store8<T, VEC>(dvp + d0, s.D - d0, dv[c]);
     }
+}
+
+// Gradient of the relative position bias: entry (n, dy, dx) is the sum of dS over every
+// (query, key) pair of head n with key - query = (dy, dx) (NATTEN's rule; the reference has
+// no bias).  One workgroup per entry walks all queries of the head in a fixed order, each
+// thread a strided share, and adds the 256 partial sums in a fixed tree: the same bits on
+// every run, where adding the pairs with atomics as they are formed does not give that.
+__global__ __launch_bounds__(256) void rpb_grad_reduce(const float *ds_pairs, float *d_rpb, Shape s) {
+    __shared__ float part[256];
+    const int EW = 2 * s.kw - 1, E = (2 * s.kh - 1) * EW;
+    const int n = blockIdx.x / E, e = blockIdx.x % E;
+    const int dy = e / EW - (s.kh - 1), dx = e % EW - (s.kw - 1);
+    const int64_t hw = (int64_t)s.H * s.W, total = (int64_t)s.B * hw;
+    float acc = 0.f;
+    for (int64_t idx = threadIdx.x; idx < total; idx += 256) {
+        const int b = (int)(idx / hw);
+        const int pix = (int)(idx % hw), x = pix / s.W, y = pix % s.W;
+        const int jx = x + dy - win_start(x, s.H, s.kh), jy = y + dx - win_start(y, s.W, s.kw);
+        if ((unsigned)jx < (unsigned)s.kh && (unsigned)jy < (unsigned)s.kw)
+            acc += ds_pairs[(((int64_t)b * s.N + n) * hw + pix) * (s.kh * s.kw) + jx * s.kw + jy];
+    }
+    part[threadIdx.x] = acc;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) part[threadIdx.x] += part[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) d_rpb[blockIdx.x] = part[0];
 }
 
 // ---------------------------------------------------------------- dispatch
@@ -439,6 +469,9 @@ int bwd_cfg(const BwdArgs &a, bool vec, hipStream_t st) {
         if (vec) hipLaunchKernelGGL((bwd_dkdv_simt<T, G, CH, true>), grid, dim3(256), 0, st, a, tx, ty);
         else hipLaunchKernelGGL((bwd_dkdv_simt<T, G, CH, false>), grid, dim3(256), 0, st, a, tx, ty);
     }
+    if (a.d_rpb)
+        hipLaunchKernelGGL(rpb_grad_reduce, dim3((unsigned)(a.s.N * (2 * a.s.kh - 1) * (2 * a.s.kw - 1))),
+                           dim3(256), 0, st, a.ds_pairs, a.d_rpb, a.s);
     return check_launch("enatten2d_bwd");
 }
 
@@ -464,7 +497,8 @@ int fwd_t(const FwdArgs &a, hipStream_t st) {
 template <typename T>
 int bwd_t(const BwdArgs &a, hipStream_t st) {
     const bool vec = a.s.D % 8 == 0 && vec_ok(a.q) && vec_ok(a.k) && vec_ok(a.v) && vec_ok(a.o) &&
-                     vec_ok(a.d_o) && vec_ok(a.dq) && vec_ok(a.dk) && vec_ok(a.dv);
+                     vec_ok(a.d_o) && vec_ok(a.dq) && vec_ok(a.dk) && vec_ok(a.dv) && a.gsb % 8 == 0 &&
+                     a.gsn % 8 == 0 && a.gsh % 8 == 0 && a.gsw % 8 == 0;
     ENATTEN_BY_D(bwd_cfg, T, a, vec, st);
 }
 

@@ -106,7 +106,9 @@ def _fwd_impl(q, k, v, kernel_size: int, scale: float, out=None):
     return o, lse
 
 
-def _bwd_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
+def _bwd_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float, out=None):
+    """`out`: (dq, dk, dv) views of one layout (unit stride on the channels) that the kernels
+    write in place (the strided sub-grids of a dilated call); None allocates them."""
     _validate(q, k, v, kernel_size)
     _require_gpu(q, "enatten::na2d_bwd")
     if d_o.shape != q.shape or o.shape != q.shape:
@@ -118,17 +120,22 @@ def _bwd_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
     lse = lse.contiguous()
     B, N, H, W, D = q.shape
     with torch.cuda.device(q.device):
-        dq = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
-        dk, dv = torch.empty_like(dq), torch.empty_like(dq)
+        if out is None:
+            dq = torch.empty((B, N, H, W, D), dtype=q.dtype, device=q.device)
+            dk, dv = torch.empty_like(dq), torch.empty_like(dq)
+        else:
+            dq, dk, dv = out
+            assert dq.stride() == dk.stride() == dv.stride() and dq.stride(-1) == 1
         ws = torch.empty(lib.enatten2d_bwd_workspace_bytes(B, N, H, W, D, kernel_size,
                                                             _DTYPES[q.dtype]),
                          dtype=torch.uint8, device=q.device)
-        _check(lib.enatten2d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                 d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                                 dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, kernel_size,
-                                 _DTYPES[q.dtype], _lib.strides4(q), _lib.strides4(k),
-                                 _lib.strides4(v), _lib.strides4(o), _lib.strides4(d_o),
-                                 float(scale), _stream_of(q)))
+        _check(lib.enatten2d_bwd_into(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                      d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                      dv.data_ptr(), ws.data_ptr(), B, N, H, W, D, kernel_size,
+                                      _DTYPES[q.dtype], _lib.strides4(q), _lib.strides4(k),
+                                      _lib.strides4(v), _lib.strides4(o), _lib.strides4(d_o),
+                                      None if out is None else _lib.strides4(dq),
+                                      float(scale), _stream_of(q)))
     return dq, dk, dv
 
 
@@ -148,7 +155,7 @@ def _fwd1d_impl(q, k, v, kernel_size: int, scale: float, out=None):
     return o, lse
 
 
-def _bwd1d_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
+def _bwd1d_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float, out=None):
     _validate(q, k, v, kernel_size, 4)
     _require_gpu(q, "enatten::na1d_bwd")
     if d_o.shape != q.shape or o.shape != q.shape:
@@ -160,16 +167,21 @@ def _bwd1d_impl(q, k, v, o, lse, d_o, kernel_size: int, scale: float):
     lse = lse.contiguous()
     B, N, T, D = q.shape
     with torch.cuda.device(q.device):
-        dq = torch.empty((B, N, T, D), dtype=q.dtype, device=q.device)
-        dk, dv = torch.empty_like(dq), torch.empty_like(dq)
+        if out is None:
+            dq = torch.empty((B, N, T, D), dtype=q.dtype, device=q.device)
+            dk, dv = torch.empty_like(dq), torch.empty_like(dq)
+        else:
+            dq, dk, dv = out
+            assert dq.stride() == dk.stride() == dv.stride() and dq.stride(-1) == 1
         ws = torch.empty(lib.enatten1d_bwd_workspace_bytes(B, N, T), dtype=torch.uint8,
                          device=q.device)
-        _check(lib.enatten1d_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                 d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                                 dv.data_ptr(), ws.data_ptr(), B, N, T, D, kernel_size,
-                                 _DTYPES[q.dtype], _lib.strides3(q), _lib.strides3(k),
-                                 _lib.strides3(v), _lib.strides3(o), _lib.strides3(d_o),
-                                 float(scale), _stream_of(q)))
+        _check(lib.enatten1d_bwd_into(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                      d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                      dv.data_ptr(), ws.data_ptr(), B, N, T, D, kernel_size,
+                                      _DTYPES[q.dtype], _lib.strides3(q), _lib.strides3(k),
+                                      _lib.strides3(v), _lib.strides3(o), _lib.strides3(d_o),
+                                      None if out is None else _lib.strides3(dq),
+                                      float(scale), _stream_of(q)))
     return dq, dk, dv
 
 
@@ -274,10 +286,8 @@ class Natten2dDilated(torch.autograd.Function):
         for i in range(dilation):
             for j in range(dilation):
                 sub = (slice(None), slice(None), slice(i, None, dilation), slice(j, None, dilation))
-                dq, dk, dv = torch.ops.enatten.na2d_bwd(Q[sub], K[sub], V[sub], o[sub],
-                                                        lses[i * dilation + j], grad_output[sub],
-                                                        kernel_size, scale)
-                dQ[sub], dK[sub], dV[sub] = dq, dk, dv
+                _bwd_impl(Q[sub], K[sub], V[sub], o[sub], lses[i * dilation + j], grad_output[sub],
+                          kernel_size, scale, out=(dQ[sub], dK[sub], dV[sub]))
         return dQ, dK, dV, None, None, None
 
 
@@ -353,9 +363,10 @@ def _window_bwd(q, k, v, rpb, o, lse, d_o, kernel, causal, scale: float):
         d_rpb = None
         if rpb is not None:
             rpb = rpb.contiguous()
-            d_rpb = torch.zeros(rpb.shape, dtype=torch.float32, device=q.device)
-        ws = torch.empty(lib.enatten2d_bwd_window_workspace_bytes(B, N, H, W), dtype=torch.uint8,
-                         device=q.device)
+            d_rpb = torch.empty(rpb.shape, dtype=torch.float32, device=q.device)
+        ws = torch.empty(lib.enatten2d_bwd_window_workspace_bytes(B, N, H, W, kernel[0], kernel[1],
+                                                                  int(rpb is not None)),
+                         dtype=torch.uint8, device=q.device)
         _check(lib.enatten2d_bwd_window(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), rpb.data_ptr() if rpb is not None else None,
             o.data_ptr(), d_o.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(),
@@ -491,9 +502,8 @@ class Natten1dDilated(torch.autograd.Function):
         dQ, dK, dV = (torch.empty(q.shape, dtype=q.dtype, device=q.device) for _ in range(3))
         for i in range(dilation):
             sub = (slice(None), slice(None), slice(i, None, dilation))
-            dq, dk, dv = torch.ops.enatten.na1d_bwd(q[sub], k[sub], v[sub], o[sub], lses[i],
-                                                    grad_output[sub], kernel_size, scale)
-            dQ[sub], dK[sub], dV[sub] = dq, dk, dv
+            _bwd1d_impl(q[sub], k[sub], v[sub], o[sub], lses[i], grad_output[sub], kernel_size,
+                        scale, out=(dQ[sub], dK[sub], dV[sub]))
         return dQ, dK, dV, None, None, None
 
 

@@ -123,6 +123,24 @@ int enatten2d_bwd(const void *q, const void *k, const void *v, const void *o,
                   void *stream);
 
 /*
+ * enatten2d_bwd that writes dq, dk and dv into strided tensors: grad_strides gives the
+ * element strides of all three on (batch, head, row, column), unit stride on the channels
+ * (NULL: contiguous, i.e. enatten2d_bwd).  It has no counterpart in the reference (whose
+ * gradients are zeros_like(Q), e_natten/triton.py:528-530); it is what lets a dilated call
+ * write the gradients of a strided sub-grid straight into the full tensors.  Strides that
+ * are no multiples of 8 elements run on the general kernels; head_dim 128 with kernel_size 5
+ * and float32 then take the two-pass / general kernels (their fused and matrix-core
+ * backward write contiguous gradients only).
+ */
+int enatten2d_bwd_into(const void *q, const void *k, const void *v, const void *o,
+                       const void *d_o, const float *lse, void *dq, void *dk, void *dv,
+                       void *workspace, int B, int heads, int H, int W, int D,
+                       int kernel_size, int dtype, const int64_t *q_strides,
+                       const int64_t *k_strides, const int64_t *v_strides,
+                       const int64_t *o_strides, const int64_t *do_strides,
+                       const int64_t *grad_strides, float scale, void *stream);
+
+/*
  * enatten2d_bwd for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  Same arguments and results as enatten2d_bwd without
@@ -158,16 +176,18 @@ int enatten2d_bwd_static(const void *q, const void *k, const void *v, const void
  * k positions up to and including its own, fewer at the start of the axis, and k may be
  * even there; on the other axes the window is the reference's
  * clamp(i - k/2, 0, L - k) with k odd.  The same conventions as enatten2d_fwd /
- * enatten2d_bwd otherwise; the workspace holds 16 bytes per query
- * (enatten2d_bwd_window_workspace_bytes: two float32, or two doubles for float64 tensors).  A 1D causal (sliding-window) attention over
+ * enatten2d_bwd otherwise; the workspace holds 16 bytes per query (two float32, or two
+ * doubles for float64 tensors) and, with a bias, kernel_h * kernel_w float32 per query more
+ * (enatten2d_bwd_window_workspace_bytes).  A 1D causal (sliding-window) attention over
  * [B, heads, T, D] is the call with H = 1, kernel_h = 1, causal_h = 0.
  *
  * rpb, NULL or a relative position bias [heads, 2 * kernel_h - 1, 2 * kernel_w - 1] of the
  * tensors' element type, contiguous: the logit of (query, key) gets entry
  * (key - query + kernel - 1) of each axis added after the scaling (NATTEN's rule; centred
- * axes only).  The backward then adds the bias gradient into d_rpb, float32 of the same
- * shape, which the caller has set to zero: it is accumulated with float atomics, so its
- * last bits can differ from run to run (dq, dk and dv stay bit-reproducible).
+ * axes only; not for float64 tensors).  The backward then writes the bias gradient to d_rpb,
+ * float32 of the same shape, fully overwritten: the dK/dV pass leaves dS of every (query,
+ * window position) in the workspace and one more kernel sums each entry's pairs in a fixed
+ * order, so d_rpb is bit-reproducible like dq, dk and dv (no atomics anywhere).
  *
  * Square, non-causal calls without a bias are handed to the kernels behind enatten2d_fwd /
  * enatten2d_bwd; everything else runs on the general kernels.
@@ -178,7 +198,8 @@ int enatten2d_fwd_window(const void *q, const void *k, const void *v, const void
                          const int64_t *q_strides, const int64_t *k_strides,
                          const int64_t *v_strides, const int64_t *o_strides, float scale,
                          void *stream);
-size_t enatten2d_bwd_window_workspace_bytes(int B, int heads, int H, int W);
+size_t enatten2d_bwd_window_workspace_bytes(int B, int heads, int H, int W, int kernel_h,
+                                            int kernel_w, int with_rpb);
 int enatten2d_bwd_window(const void *q, const void *k, const void *v, const void *rpb,
                          const void *o, const void *d_o, const float *lse, void *dq, void *dk,
                          void *dv, float *d_rpb, void *workspace, int B, int heads, int H, int W,
@@ -208,6 +229,15 @@ int enatten1d_bwd(const void *q, const void *k, const void *v, const void *o,
                   int dtype, const int64_t *q_strides, const int64_t *k_strides,
                   const int64_t *v_strides, const int64_t *o_strides,
                   const int64_t *do_strides, float scale, void *stream);
+/* enatten1d_bwd with dq, dk, dv written through grad_strides (batch, head, position), as
+ * enatten2d_bwd_into */
+int enatten1d_bwd_into(const void *q, const void *k, const void *v, const void *o,
+                  const void *d_o, const float *lse, void *dq, void *dk, void *dv,
+                  void *workspace, int B, int heads, int T, int D, int kernel_size,
+                  int dtype, const int64_t *q_strides, const int64_t *k_strides,
+                  const int64_t *v_strides, const int64_t *o_strides,
+                  const int64_t *do_strides, const int64_t *grad_strides,
+                       float scale, void *stream);
 
 /*
  * Per-kernel timing aid for benchmarks (no counterpart in the reference, whose

@@ -214,7 +214,8 @@ def test_window_entry_points_validate(lib):
     assert f(3, 0, 0, 1) == 1
     assert f(3, 4, 0, 1, q=None) == 1 and "q is NULL" in _lib.last_error()   # even is fine when causal
     assert f(4, 4) == 1 and "odd" in _lib.last_error()   # square non-causal: the plain entry point's rule
-    assert lib.enatten2d_bwd_window_workspace_bytes(2, 3, 4, 5) == 2 * 3 * 4 * 5 * 16
+    assert lib.enatten2d_bwd_window_workspace_bytes(2, 3, 4, 5, 3, 7, 0) == 2 * 3 * 4 * 5 * 16
+    assert lib.enatten2d_bwd_window_workspace_bytes(2, 3, 4, 5, 3, 7, 1) == 2 * 3 * 4 * 5 * (16 + 21 * 4)
     assert f(3, 5, 0, 1, rpb=1) == 1 and "centred axes only" in _lib.last_error()
     assert lib.enatten2d_bwd_window(1, 1, 1, None, 1, 1, None, 1, 1, 1, None, None, 1, 1, 8, 8, 16, 3, 5,
                                     0, 0, 0, None, None, None, None, None, 1.0, None) == 1
