@@ -204,6 +204,8 @@ def main():
     ap.add_argument("--seq", type=int, default=0,
                     help="time natten1d on [batch, heads, SEQ, head_dim] sequences instead of "
                          "natten2d on images (no sweep, no unfused comparator, no CPU baseline)")
+    ap.add_argument("--event-period", type=int, default=0,
+                    help="bracket every N-th launch of each kernel with HIP events (default: steps // 10)")
     ap.add_argument("--config", choices=sorted(CONFIGS),
                     help="one of the named benchmark configurations (sets the shape flags)")
     args = ap.parse_args()
@@ -249,9 +251,9 @@ def main():
         step(i)
     torch.cuda.synchronize()
     # Per-kernel HIP events inside the timed region: every `period`-th launch of
-    # each kernel is bracketed (a record costs ~3 us of queue time; timing all of
-    # them would stretch the step by ~10%).
-    period = max(1, args.steps // 10)
+    # each kernel is bracketed (a record costs ~5 us of queue time; timing all of
+    # them would stretch the step by ~7%).
+    period = args.event_period if args.event_period > 0 else max(1, args.steps // 10)
     lib.enatten_profile_enable(period)
     t0 = time.perf_counter()
     for i in range(args.steps):
@@ -318,9 +320,15 @@ def main():
         lib.enatten_profile_read(i, ctypes.byref(n), ctypes.byref(tot))
         if n.value == 0:
             continue
-        avg_ms = tot.value / n.value
+        empty = ctypes.c_double()
+        lib.enatten_profile_read_overhead(i, ctypes.byref(empty))
+        raw_us, empty_us = tot.value / n.value * 1e3, empty.value / n.value * 1e3
+        # avg_us: the bracket's reading less what the bracket itself adds (an event recorded
+        # straight after the closing one, nothing in between, measures that on the same
+        # busy queue).  Uncorrected, the brackets of one step sum to more than its wall time.
         kern[name] = {"kernel": lib.enatten_profile_kernel_name(i).decode(), "launches": n.value,
-                      "avg_us": avg_ms * 1e3, "alg_bytes": alg.get(name, 0)}
+                      "avg_us": raw_us - empty_us, "bracket_us": raw_us, "empty_bracket_us": empty_us,
+                      "alg_bytes": alg.get(name, 0)}
     for k in kern.values():
         k["GBps"] = k["alg_bytes"] / (k["avg_us"] * 1e-6) / 1e9
     names = list(kern)
@@ -363,7 +371,8 @@ def main():
         "working_set_fits_memory_side_cache": working_set <= MALL_BYTES,
         "host_enqueue_ms_per_step": host_s * 1e3 / args.steps,
         "graph_replay_ms_per_step": graph_ms,
-        "kernel_event_sampling": "every %d-th launch" % period,
+        "kernel_event_sampling": "every %d-th launch; avg_us = bracket_us - empty_bracket_us "
+                                 "(an event pair with nothing between, recorded after each bracket)" % period,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": ("natten1d fwd+bwd B=%d heads=%d T=%d head_dim=%d kernel_size=%d"

@@ -40,6 +40,7 @@ SIGNATURES = {
     "enatten1d_bwd_into": (_i, [_vp] * 10 + [_i] * 6 + [_sp] * 6 + [ctypes.c_float, _vp]),
     "enatten_profile_enable": (_i, [_i]),
     "enatten_profile_read": (_i, [_i, ctypes.POINTER(_i), ctypes.POINTER(ctypes.c_double)]),
+    "enatten_profile_read_overhead": (_i, [_i, ctypes.POINTER(ctypes.c_double)]),
     "enatten_profile_kernel_name": (ctypes.c_char_p, [_i]),
 }
 

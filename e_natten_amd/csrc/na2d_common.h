@@ -100,7 +100,7 @@ void set_error(const char *fmt, ...);
 struct ProfScope {
     int slot;
     hipStream_t st;
-    hipEvent_t e0, e1;
+    hipEvent_t e0, e1, e2;
     unsigned generation;
     bool armed;
     ProfScope(int kernel_slot, const char *kernel_name, hipStream_t stream);

@@ -258,6 +258,12 @@ enum { ENATTEN_KERNEL_FWD = 0, ENATTEN_KERNEL_BWD_DQ = 1, ENATTEN_KERNEL_BWD_DKD
        ENATTEN_KERNEL_BWD_FUSED = 3, ENATTEN_KERNEL_COUNT = 4 };
 int enatten_profile_enable(int on);
 int enatten_profile_read(int kernel, int *launches, double *total_ms);
+/* What the brackets themselves added to total_ms: after each timed launch's closing
+ * event a further event is recorded with nothing in between, and the time between
+ * those two (the cost of one event on a busy queue, about 5 us on MI355X) is summed
+ * here over the same launches.  total_ms minus this is the kernels' own time; without
+ * the correction the brackets of one step add up to more than the step's wall time. */
+int enatten_profile_read_overhead(int kernel, double *total_empty_ms);
 /* Name of the device kernel last launched for that slot ("" if none yet). */
 const char *enatten_profile_kernel_name(int kernel);
 
