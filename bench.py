@@ -204,6 +204,10 @@ def main():
     ap.add_argument("--seq", type=int, default=0,
                     help="time natten1d on [batch, heads, SEQ, head_dim] sequences instead of "
                          "natten2d on images (no sweep, no unfused comparator, no CPU baseline)")
+    ap.add_argument("--spin-up-ms", type=float, default=60.0,
+                    help="untimed steps of the same workload for this long before the warm-up steps: "
+                         "from idle the GPU needs ~20 ms of load to settle (steps take 190, then "
+                         "200-218, then 182 us at the default shape)")
     ap.add_argument("--event-period", type=int, default=0,
                     help="bracket every N-th launch of each kernel with HIP events (default: steps // 10)")
     ap.add_argument("--config", choices=sorted(CONFIGS),
@@ -247,6 +251,15 @@ def main():
         o = op(q, k, v, ks)
         return torch.autograd.grad(o, (q, k, v), d_o)
 
+    step(0)   # (the first call loads code objects and queries occupancies: not part of the spin-up)
+    torch.cuda.synchronize()
+    spin_steps = 0
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < args.spin_up_ms:
+        for i in range(32):
+            step(spin_steps + i)
+        torch.cuda.synchronize()
+        spin_steps += 32
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -365,6 +378,8 @@ def main():
                   % ("natten1d" if args.seq else "natten2d", B, N, D, ks, args.dtype),
         "value": useful / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "spin_up": "%d untimed steps (%.0f ms) before the warm-up steps, so that the timed steps see "
+                   "the GPU's settled clocks" % (spin_steps, args.spin_up_ms),
         "timing": "cold: %d input sets in rotation (%s twice the 256 MB memory-side cache)"
                   % (len(sets), "more than" if cold else "LESS than"),
         "hot_ms_per_step": hot_ms,
