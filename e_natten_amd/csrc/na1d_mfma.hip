@@ -8,7 +8,7 @@
 // kernel_size <= 49.  The rows of K and V that the tile needs (64 + k - 1 positions)
 // are staged in LDS once per tile with coalesced 16-byte loads; the next tile's rows
 // are in flight into registers while the current one is computed.  Everything else is
-// the scheme of the 2D kernels (na2d_mfma.hip): every lane holds the logits of one
+// the scheme of the 2D kernels (na2d_mfma_kernels.h): every lane holds the logits of one
 // query for several keys, the reduction index of the second product is enumerated in
 // the order the accumulators hold it, and its other operand comes out of LDS through
 // the transposing read.  The kernel size is a run-time argument: a token's place in

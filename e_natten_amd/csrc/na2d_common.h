@@ -131,6 +131,9 @@ int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st);
 // `path`: 0 chooses between the two-pass and the fused backward, ENATTEN_PATH_MFMA_FUSED /
 // ENATTEN_PATH_MFMA_SPLIT force one of them
 int launch_bwd_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st);
+// the same kernels built for head dims that are multiples of 8 below the next of 32, 64, 128
+int launch_fwd_mfma_narrow(const FwdArgs &a, int dtype, hipStream_t st);
+int launch_bwd_mfma_narrow(const BwdArgs &a, int dtype, int path, hipStream_t st);
 // matrix-core kernels of the 1D operator (a.s: H = 1, W = T, kh = 1, kw = kernel_size):
 // bf16 / f16, D in {32, 64, 128}, odd kernel_size 3 .. 49
 bool mfma1d_supported(int D, int ks, int dtype);

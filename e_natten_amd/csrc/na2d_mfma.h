@@ -116,10 +116,12 @@ __device__ __forceinline__ void store16(short *p, u32x4 v) {
 // runs).  So at D = 128 the four lanes of a token first exchange pieces with
 // v_permlane*_swap (a 4x4 transpose between lane group g and piece number j), and store
 // j of the four lanes then covers 64 contiguous bytes.  Every lane of the wave
-// must call this; `live` says whether this lane's token exists.
+// must call this; `live` says whether this lane's token exists.  `dlim` is the tensor's
+// head dim where it is narrower than the D the kernel is built for (a multiple of 8):
+// pieces at or beyond it are not stored.
 template <bool BF, int D>
 __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *acc, float mul,
-                                            bool live) {
+                                            bool live, int dlim = D) {
     constexpr int NP = D / 32;
     u32x4 p[NP];
 #pragma unroll
@@ -157,7 +159,7 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
         if (live) {
 #pragma unroll
             for (int j = 0; j < NP; j++)
-                store16(token + j * (D / 4) + g * 8, p[j]);
+                if (j * (D / 4) + g * 8 < dlim) store16(token + j * (D / 4) + g * 8, p[j]);
         }
     } else {
         // D = 32: the four lanes of a token already cover its 64 bytes.  D = 64 (pieces
@@ -165,8 +167,22 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
         if (live) {
 #pragma unroll
             for (int j = 0; j < NP; j++)
-                store16(token + g * (D / 4) + j * 8, p[j]);
+                if (g * (D / 4) + j * 8 < dlim) store16(token + g * (D / 4) + j * 8, p[j]);
         }
+    }
+}
+
+// B operand rows straight from global memory: lane group g takes channels ds*32 + g*8 ..
+// of the row at `row` (its channel 0) for ds = 0 .. DS-1.  Chunks at or beyond `dlim`
+// (head dims narrower than the kernel's D) are zero and read nothing out of bounds.
+template <int DS>
+__device__ __forceinline__ void load_row_chunks(s16x8 (&reg)[DS], const short *row, int g, int dlim) {
+#pragma unroll
+    for (int ds = 0; ds < DS; ds++) {
+        const int ch = ds * 32 + g * 8;
+        const bool on = ch < dlim;
+        const s16x8 v = *reinterpret_cast<const s16x8 *>(row + (on ? ch : 0));
+        reg[ds] = on ? v : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
 }
 
@@ -384,13 +400,16 @@ struct HaloPlan {
     int rc[Geo<D, KS, NW, SP>::NL];  // halo row << 8 | halo column of chunk i
     int ch8;                 // first channel of the thread's chunks
     int lds0;                // LDS element offset of chunk 0
+    bool on;                 // false: the tensor has no such channels (head dim below D); the
+                             // thread moves nothing and its LDS columns stay zero (zero_row)
 };
 template <int D, int KS, int NW = 4, int SP = 1>
-__device__ __forceinline__ HaloPlan<D, KS, NW, SP> make_plan() {
+__device__ __forceinline__ HaloPlan<D, KS, NW, SP> make_plan(int dlim = D) {
     using G = Geo<D, KS, NW, SP>;
     static_assert(G::NT % G::CPR == 0, "a thread keeps one channel chunk");
     HaloPlan<D, KS, NW, SP> pl;
     pl.ch8 = (threadIdx.x % G::CPR) * 8;
+    pl.on = pl.ch8 < dlim;
     // the rows of one thread's chunks are NT / CPR apart, a multiple of 16 * RPL, so they
     // share one key and the chunk position is the same for all of them
     static_assert((G::NT / G::CPR) % (16 * G::RPL) == 0, "one chunk position per thread");
@@ -421,6 +440,7 @@ __device__ __forceinline__ void halo_fetch(HaloRegs<D, KS, NW, SP> &reg, const H
     const char *base = reinterpret_cast<const char *>(img + hr0 * sh + hc0 * sw);
     const unsigned sh2 = (unsigned)sh * 2u, sw2 = (unsigned)sw * 2u;
     const int rmax = rlim - 1 - hr0, cmax = clim - 1 - hc0;
+    if (!pl.on) return;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
         const unsigned r = (unsigned)min(pl.rc[i] >> 8, rmax);
@@ -434,6 +454,7 @@ template <int D, int KS, int NW = 4, int SP = 1>
 __device__ __forceinline__ void halo_commit(short *lds, const HaloPlan<D, KS, NW, SP> &pl,
                                    const HaloRegs<D, KS, NW, SP> &reg) {
     using G = Geo<D, KS, NW, SP>;
+    if (!pl.on) return;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
         const int row = threadIdx.x / G::CPR + i * (G::NT / G::CPR);
@@ -454,6 +475,7 @@ __device__ __forceinline__ void halo_fetch_rows(HaloRegs<D, KS, NW, SP> &reg, co
     const char *base = reinterpret_cast<const char *>(img + yb * sh + hc0 * sw);
     const unsigned sh2 = (unsigned)sh * 2u, sw2 = (unsigned)sw * 2u;
     const int rmax = rlim - 1 - yb, cmax = clim - 1 - hc0;
+    if (!pl.on) return;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
         const int r = pl.rc[i] >> 8;
@@ -470,6 +492,7 @@ __device__ __forceinline__ void halo_commit_rows(short *lds, const HaloPlan<D, K
                                                  const HaloRegs<D, KS, NW, SP> &reg, int y0, int nrows) {
     using G = Geo<D, KS, NW, SP>;
     const int rot = y0 % G::HR;
+    if (!pl.on) return;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
         const int pix = threadIdx.x / G::CPR + i * (G::NT / G::CPR);
@@ -484,12 +507,22 @@ __device__ __forceinline__ void halo_commit_rows(short *lds, const HaloPlan<D, K
 }
 // The spare row stays zero for the whole kernel: padding tokens and tokens
 // outside a wave's halo read it, so they add exact zeros to the second product.
+// With a head dim below D (`dlim`), the channels from it on are zeroed in EVERY row, once:
+// no commit writes them (HaloPlan::on), so they stay zero as long as nothing else is laid
+// over the rows.
 template <int D, int KS, int NW = 4, int SP = 1>
-__device__ __forceinline__ void zero_row(short *lds) {
+__device__ __forceinline__ void zero_row(short *lds, int dlim = D) {
     using G = Geo<D, KS, NW, SP>;
     if (threadIdx.x < G::CPR)
         *reinterpret_cast<uint4 *>(lds + G::ZROW * G::PITCH + threadIdx.x * 8) =  // all zero: any order
             make_uint4(0, 0, 0, 0);
+    if (dlim < D) {
+        static_assert(!G::SWZ, "the padding columns are the last chunks of a row");
+        const int c0 = dlim >> 3, npad = G::CPR - c0;
+        for (int idx = threadIdx.x; idx < G::ZROW * npad; idx += G::NT)
+            *reinterpret_cast<uint4 *>(lds + (idx / npad) * G::PITCH + (c0 + idx % npad) * 8) =
+                make_uint4(0, 0, 0, 0);
+    }
 }
 
 // What one lane needs to know about its query (forward, dQ) inside a tile.

@@ -1,7 +1,7 @@
 // Fused backward of 2D neighborhood attention on the matrix cores of gfx950:
 // dQ, dK and dV of an 8x8 tile of pixels from ONE staging of the tile's
 // (8+k-1)^2 block of q, k, v and dO, so that the backward reads each input once
-// (the two passes of na2d_mfma.hip read them twice).
+// (the two passes of na2d_mfma_kernels.h read them twice).
 //
 // A workgroup is eight waves around one copy of the block in LDS (all four
 // tensors, which is why only one workgroup fits a CU):
@@ -12,7 +12,7 @@
 // Both sides recompute P from the saved log-sum-exp.  delta = dO . O of the block's
 // queries is formed while the block is written to LDS (the forward output is read
 // for this and for nothing else).  The MFMA operand layouts, the token numbering
-// and the transposing LDS reads are those of na2d_mfma.hip.
+// and the transposing LDS reads are those of na2d_mfma_kernels.h.
 //
 // The block of the tile at (r0, c0) is the pixels [r0 - k/2, r0 + 8 + k/2) x
 // [c0 - k/2, c0 + 8 + k/2); with image sides that are multiples of 8 it holds

@@ -2,7 +2,7 @@
 // configurations whose staged block of ALL four inputs fits LDS at least twice per CU
 // (head_dim 32 with kernel_size 3, 5, 7; head_dim 64 with kernel_size 3): dQ, dK and dV of an
 // 8x8 tile of pixels from one staging of the tile's (8+k-1)^2 block of q, k, v and dO, so
-// that the backward reads every input once where the two passes of na2d_mfma.hip read them
+// that the backward reads every input once where the two passes of na2d_mfma_kernels.h read them
 // twice (the reference's backward is one kernel too, e_natten/triton.py:304-423, with atomics
 // where this one gathers over the inverse neighbourhood).
 //
@@ -12,7 +12,7 @@
 // them (the inverse neighbourhood of e_natten/pytorch.py:13-23, :261-288), all operands out
 // of LDS.  delta = dO . O of every staged query is formed while the block is written to LDS
 // (the forward output is read for this alone).  Operand layouts, token numbering and the
-// transposing LDS reads are those of na2d_mfma.hip; this is the 2D twin of bwd1d_fused_mfma.
+// transposing LDS reads are those of na2d_mfma_kernels.h; this is the 2D twin of bwd1d_fused_mfma.
 //
 // Tiles and blocks for any image with sides >= 8: tile origins are min(8 t, L - 8) on each
 // axis (the last tile is shifted back to end with the image), and a pixel in the last 8 rows

@@ -367,6 +367,53 @@ def test_output_written_into_callers_layout(shape, ks, _lib):
     assert_close(got, (ref[0], ref[2], ref[3], ref[4]), BF, "O in the caller's layout")
 
 
+@pytest.mark.parametrize("D,ks,hw,dtype", [
+    (8, 3, (16, 16), BF), (16, 5, (24, 19), BF), (16, 13, (17, 32), F16), (24, 7, (16, 24), BF),
+    (40, 5, (32, 32), BF), (48, 5, (40, 33), BF), (48, 9, (24, 40), F16), (56, 7, (19, 17), BF),
+    (72, 3, (16, 16), BF), (80, 5, (32, 24), BF), (96, 7, (24, 24), F16), (96, 13, (32, 20), BF),
+    (104, 9, (18, 23), BF), (120, 5, (48, 40), BF), (112, 11, (20, 20), BF),
+])
+def test_head_dims_between_the_built_ones(D, ks, hw, dtype, _lib):
+    """Head dims that are multiples of 8 run on the matrix-core kernels of the next of 32, 64,
+    128 (zero channels in LDS, the stores leave them out).  Through the C ABI, every tensor a
+    [.., D] view of a buffer with 8 more channels per pixel that hold NaN (inputs) or a marker
+    (outputs): the results match the oracle and not one guard channel is read or written."""
+    from e_natten_amd import _lib as L, kernel_path
+    assert kernel_path(D, ks, dtype) == "mfma"
+    B, N, (H, W) = 2, 3, hw
+    shape = (B, N, H, W, D)
+    code = {BF: L.BF16, F16: L.F16}[dtype]
+    q, k, v, g = make_inputs(shape, dtype, 40 + D)
+    print("case narrow head dim", shape, dtype, "k=%d" % ks, flush=True)
+    ref = oracle_all(q, k, v, g, ks, small=True)
+    dev = torch.device("cuda:0")
+
+    def guarded(t=None):
+        buf = torch.full(shape[:-1] + (D + 8,), float("nan") if t is not None else 512.0, dtype=dtype, device=dev)
+        if t is not None:
+            buf[..., :D].copy_(t.to(dev))
+        return buf, buf[..., :D]
+
+    (_, qv), (_, kv), (_, vv), (_, gv) = (guarded(t) for t in (q, k, v, g))
+    (ob, ov), (dqb, dqv), (dkb, dkv), (dvb, dvv) = (guarded() for _ in range(4))
+    lse = torch.empty((B, N, H, W), dtype=torch.float32, device=dev)
+    ws = torch.empty(_lib.enatten2d_bwd_workspace_bytes(B, N, H, W, D, ks, code), dtype=torch.uint8, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    sq, sk, sv, sg, so, sgr = (L.strides4(t) for t in (qv, kv, vv, gv, ov, dqv))
+    rc = _lib.enatten2d_fwd(qv.data_ptr(), kv.data_ptr(), vv.data_ptr(), ov.data_ptr(), lse.data_ptr(),
+                            B, N, H, W, D, ks, code, sq, sk, sv, so, 1.0, st)
+    assert rc == 0, L.last_error()
+    rc = _lib.enatten2d_bwd_into(qv.data_ptr(), kv.data_ptr(), vv.data_ptr(), ov.data_ptr(), gv.data_ptr(),
+                                 lse.data_ptr(), dqv.data_ptr(), dkv.data_ptr(), dvv.data_ptr(), ws.data_ptr(),
+                                 B, N, H, W, D, ks, code, sq, sk, sv, so, sg, sgr, 1.0, st)
+    assert rc == 0, L.last_error()
+    torch.cuda.synchronize()
+    for name, buf in (("O", ob), ("dQ", dqb), ("dK", dkb), ("dV", dvb)):
+        assert (buf[..., D:].float() == 512.0).all(), "%s: a guard channel was written" % name
+    got = tuple(t.float().cpu() for t in (ov, dqv, dkv, dvv))
+    assert_close(got, (ref[0], ref[2], ref[3], ref[4]), dtype, "head_dim %d k%d" % (D, ks))
+
+
 @pytest.mark.parametrize("D,ks", [(128, 5), (64, 7), (32, 3)])
 def test_misaligned_views_take_the_general_kernels(D, ks, _lib):
     # head dims the matrix-core kernels serve, but as views whose rows are not 16-byte

@@ -66,6 +66,10 @@ def test_kernel_path_query(lib):
     # every kernel size of the matrix-core kernels at head_dim 128, the largest windows included
     assert all(kernel_path(128, ks, torch.bfloat16) == "mfma" for ks in (3, 5, 7, 9, 11, 13))
     assert kernel_path(128, 13, torch.float16) == "mfma" and kernel_path(128, 15, torch.bfloat16) == "simt"
+    # multiples of 8 below the built head dims run on the next one's kernels (not 64 with k 11, 13)
+    assert all(kernel_path(d, 5, torch.bfloat16) == "mfma" for d in (8, 16, 24, 40, 48, 56, 72, 96, 120))
+    assert kernel_path(48, 13, torch.bfloat16) == "simt" and kernel_path(96, 13, torch.float16) == "mfma"
+    assert kernel_path(20, 5, torch.bfloat16) == "simt" and kernel_path(256, 5, torch.bfloat16) == "simt"
     assert kernel_path(2, 3, torch.float32) == "simt"
     assert kernel_path(128, 4, torch.bfloat16) == "none"
     assert kernel_path(4096, 3, torch.bfloat16) == "none"
