@@ -55,6 +55,29 @@ def test_random_shapes_2d(shape, ks, dtype, path, scale, seed, lib):
         lib.enatten_set_path(prev)
 
 
+def _cases_2d_narrow(n, seed):
+    """Head dims that are multiples of 8 between the built ones (matrix-core kernels of the next
+    of 32, 64, 128; head dims below 64 with kernel_size 11 and 13 take the general kernels)."""
+    rnd = random.Random(seed)
+    out = []
+    for it in range(n):
+        dt = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+        D = rnd.choice([8, 16, 24, 40, 48, 56, 72, 80, 88, 96, 104, 112, 120])
+        ks = rnd.choice([3, 5, 5, 7, 7, 9, 11, 13])
+        H, W = rnd.randint(ks, 60), rnd.randint(ks, 60)
+        if rnd.random() < 0.4:
+            H, W = max(ks, (H + 7) // 8 * 8), max(ks, (W + 7) // 8 * 8)
+        B = rnd.choice([1, 2, 3])
+        N = max(1, int(rnd.choice([2e4, 8e4, 2e5]) / (H * W)) // B)
+        out.append(((B, N, H, W, D), ks, dt, rnd.choice([0, 0, 3, 4]), rnd.choice([1.0, 0.5, D ** -0.5]), it))
+    return out
+
+
+@pytest.mark.parametrize("shape,ks,dtype,path,scale,seed", _cases_2d_narrow(20, 31))
+def test_random_shapes_2d_narrow_head_dims(shape, ks, dtype, path, scale, seed, lib):
+    test_random_shapes_2d(shape, ks, dtype, path, scale, 1000 + seed, lib)
+
+
 def _cases_1d(n, seed):
     rnd = random.Random(seed)
     out = []
