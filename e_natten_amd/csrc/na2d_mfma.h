@@ -119,7 +119,14 @@ __device__ __forceinline__ void store16(short *p, u32x4 v) {
 // must call this; `live` says whether this lane's token exists.  `dlim` is the tensor's
 // head dim where it is narrower than the D the kernel is built for (a multiple of 8):
 // pieces at or beyond it are not stored.
-template <bool BF, int D>
+// LINES (D = 128 only): one more exchange, between the lanes of tokens n and n^1, after which
+// every store instruction writes whole 128-byte lines (see below).  It removes the 8-10% of
+// extra HBM writes of the 64-byte runs (forward 73.1 -> 68.2 MB, dQ pass 73.5 -> 68.2, dK/dV
+// 148.6 -> 134.2, fused backward 222.8 -> 201.4 at B4 N4 128x128) and is used by the kernels
+// that run two workgroups per CU, which get 1-9% faster with it (forward 203 -> 194 us at
+// 256x256, dQ pass 61.8 -> 56.2, dK/dV 92.6 -> 86.7); the kernels with one workgroup per CU
+// get slower (fused backward 118 -> 139 us, dK/dV at k = 7 153 -> 165) and keep the 64-byte runs.
+template <bool BF, int D, bool LINES = false>
 __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *acc, float mul,
                                             bool live, int dlim = D) {
     constexpr int NP = D / 32;
@@ -156,7 +163,44 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
                 p[2 * j1 + 1][c] = r[1];
             }
         // piece j of this lane is now channels j*D/4 + g*8 .. +8
-        if (live) {
+        if constexpr (LINES) {
+            // Stored like that, an instruction would write 64 contiguous bytes per token: half a
+            // line, and non-temporal half lines leave L2 before their other half arrives (a pure
+            // write stream of 64-byte runs moves 1.42x its bytes at 3.1 TB/s, one of 128-byte runs
+            // 1.00x at 5.3 TB/s).  So the lanes of tokens n and n^1 (adjacent lanes) exchange once
+            // more: the even lane gives pieces 1 and 3 and takes the odd lane's 0 and 2, and the
+            // eight lanes of the pair then write one token's line per instruction.
+            const bool odd = threadIdx.x & 1;
+            auto xchg = [](unsigned x) __attribute__((always_inline)) {
+                return (unsigned)__builtin_amdgcn_mov_dpp((int)x, 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true);
+            };
+            u32x4 s0, s1, s2, s3;
+    #pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const unsigned ra = xchg(odd ? p[0][c] : p[1][c]), rb = xchg(odd ? p[2][c] : p[3][c]);
+                s0[c] = odd ? ra : p[0][c];
+                s1[c] = odd ? rb : p[2][c];
+                s2[c] = odd ? p[1][c] : ra;
+                s3[c] = odd ? p[3][c] : rb;
+            }
+            // (the other token's address as an offset from this one's, so that the stores stay
+            // global-memory instructions: an address rebuilt from exchanged integers makes them flat)
+            const uintptr_t own = reinterpret_cast<uintptr_t>(token);
+            const uintptr_t nbr = (uintptr_t)xchg((unsigned)own) | ((uintptr_t)xchg((unsigned)(own >> 32)) << 32);
+            const bool nlive = xchg(live ? 1u : 0u) != 0;
+            short *other = reinterpret_cast<short *>(reinterpret_cast<char *>(token) + (ptrdiff_t)(nbr - own));
+            short *tok_a = odd ? other : token, *tok_b = odd ? token : other;
+            const bool live_a = odd ? nlive : live, live_b = odd ? live : nlive;
+            const int off = (odd ? 32 : 0) + g * 8;
+            if (live_a) {
+                if (off < dlim) store16(tok_a + off, s0);
+                if (off + 64 < dlim) store16(tok_a + off + 64, s1);
+            }
+            if (live_b) {
+                if (off < dlim) store16(tok_b + off, s2);
+                if (off + 64 < dlim) store16(tok_b + off + 64, s3);
+            }
+        } else if (live) {
 #pragma unroll
             for (int j = 0; j < NP; j++)
                 if (j * (D / 4) + g * 8 < dlim) store16(token + j * (D / 4) + g * 8, p[j]);
