@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256, 2) void fwd1d_mfma(FwdArgs a, int tiles_t, int
                     o[mt] = mfma16<BF>(cat(lds_read_tr(vp[0] + mt * 4), lds_read_tr(vp[1] + mt * 4)),
                                        pb[kk], o[mt]);
             }
-            store_token<BF, D, D == 128>(const_cast<short *>(seq(a.o, cur)) + lq.qt * a.o.sw, g, o, 1.f / sum,
+            store_token<BF, D, D >= 64>(const_cast<short *>(seq(a.o, cur)) + lq.qt * a.o.sw, g, o, 1.f / sum,
                                lq.live);
             if (lq.live && a.lse && g == 0) a.lse[lq.tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
         }
@@ -318,7 +318,7 @@ __global__ __launch_bounds__(256, 2) void bwd1d_dq_mfma(BwdArgs a, int tiles_t, 
                     dq[mt] = mfma16<BF>(cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)),
                                         dsb[kk], dq[mt]);
             }
-            store_token<BF, D, D == 128>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, 0, lq.qt), g, dq, s.scale, lq.live);
+            store_token<BF, D, D >= 64>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, 0, lq.qt), g, dq, s.scale, lq.live);
             if (lq.live && g == 0) a.delta[lq.tok] = delta;
         }
         if (!more) break;
@@ -446,8 +446,8 @@ __global__ __launch_bounds__(256, 2) void bwd1d_dkdv_mfma(BwdArgs a, int tiles_t
             }
             const int64_t goff = a.grad_at(cur.bb, cur.nn, 0, kt);
             const bool live = w0 + n < T;
-            store_token<BF, D, D == 128>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live);
-            store_token<BF, D, D == 128>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live);
+            store_token<BF, D, D >= 64>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live);
+            store_token<BF, D, D >= 64>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live);
         }
         if (!more) break;
         load_keys(nxt);
@@ -586,7 +586,7 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
                         dq[mt] = mfma16<BF>(cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)),
                                             dsb[kk], dq[mt]);
                 }
-                store_token<BF, D>(static_cast<short *>(a.dq) + goff, g, dq, s.scale, live);
+                store_token<BF, D, D == 64>(static_cast<short *>(a.dq) + goff, g, dq, s.scale, live);
             }
             {
                 // ---- dK, dV: the queries that attend to any of the wave's 16 keys, 32 at a time
@@ -643,8 +643,8 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
                         dk[mt] = mfma16<BF>(cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)), dsb, dk[mt]);
                     }
                 }
-                store_token<BF, D>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live);
-                store_token<BF, D>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live);
+                store_token<BF, D, D == 64>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live);
+                store_token<BF, D, D == 64>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live);
             }
         }
         if (!more) break;

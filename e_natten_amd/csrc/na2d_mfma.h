@@ -205,9 +205,30 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
             for (int j = 0; j < NP; j++)
                 if (j * (D / 4) + g * 8 < dlim) store16(token + j * (D / 4) + g * 8, p[j]);
         }
+    } else if constexpr (NP == 2 && LINES) {
+        // D = 64: a lane holds 32 contiguous bytes of its token (two pieces), so an instruction
+        // writes 16-byte pieces 32 bytes apart.  The lanes of tokens n and n^1 exchange one piece
+        // each and the eight lanes of the pair write one token's whole line per instruction.
+        const bool odd = threadIdx.x & 1;
+        auto xchg = [](unsigned x) __attribute__((always_inline)) {
+            return (unsigned)__builtin_amdgcn_mov_dpp((int)x, 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true);
+        };
+        u32x4 s0, s1;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const unsigned r = xchg(odd ? p[0][c] : p[1][c]);
+            s0[c] = odd ? r : p[0][c];
+            s1[c] = odd ? p[1][c] : r;
+        }
+        const uintptr_t own = reinterpret_cast<uintptr_t>(token);
+        const uintptr_t nbr = (uintptr_t)xchg((unsigned)own) | ((uintptr_t)xchg((unsigned)(own >> 32)) << 32);
+        const bool nlive = xchg(live ? 1u : 0u) != 0;
+        short *other = reinterpret_cast<short *>(reinterpret_cast<char *>(token) + (ptrdiff_t)(nbr - own));
+        const int off = g * 16 + (odd ? 8 : 0);
+        if ((odd ? nlive : live) && off < dlim) store16((odd ? other : token) + off, s0);
+        if ((odd ? live : nlive) && off < dlim) store16((odd ? token : other) + off, s1);
     } else {
-        // D = 32: the four lanes of a token already cover its 64 bytes.  D = 64 (pieces
-        // 32 bytes apart): the corresponding exchange was measured and gains nothing.
+        // D = 32: the four lanes of a token already cover its 64 bytes.
         if (live) {
 #pragma unroll
             for (int j = 0; j < NP; j++)

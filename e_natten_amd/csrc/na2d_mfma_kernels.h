@@ -41,10 +41,14 @@
 namespace enatten {
 namespace {
 
-// Whole-line stores (store_token's LINES) where a kernel runs two workgroups per CU on
-// tensors of head_dim 128 itself (tokens are then two aligned lines each).
-template <int D, int WGS>
-constexpr bool kLineStores = D == 128 && !kNarrow && WGS == 2;
+// Whole-line stores (store_token's LINES) where a kernel runs at least two workgroups per CU
+// on tensors of head_dim 128 or 64 itself (a token is then two aligned lines, or one).
+// Measured, us, without -> with: d = 128 see store_token; d = 64 B4 N8 128x128 k5 forward 65.4 ->
+// 61.4, dQ 67.8 -> 65.5, dK/dV 83.7 -> 76.1; B4 N4 256x256 k5 473 -> 427 per forward+backward;
+// k7 284 -> 282; no gain from k = 9 on (343 -> 347, 281.4 -> 280.9 at k13), where the kernels
+// do not wait for their stores, so it stops at 7 there.
+template <int D, int KS, int WGS>
+constexpr bool kLineStores = (D == 128 || (D == 64 && KS <= 7)) && !kNarrow && WGS >= 2;
 
 // ------------------------------------------------------------------ forward
 // ROLL: walk down the columns of an image and keep the halo rows that consecutive
@@ -171,7 +175,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
                         o[mt]);
             }
 
-            store_token<BF, D, kLineStores<D, G::WAVES>>(const_cast<short *>(image<short>(a.o, cur)) + lq.qr * a.o.sh + lq.qc * a.o.sw,
+            store_token<BF, D, kLineStores<D, KS, G::WAVES>>(const_cast<short *>(image<short>(a.o, cur)) + lq.qr * a.o.sh + lq.qc * a.o.sw,
                                g, o, 1.f / sum, lq.live, dlim);
             if (lq.live && a.lse && g == 0)
                 a.lse[lq.tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
@@ -298,7 +302,7 @@ __global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void fwd2_mfma(FwdArgs a
                         cat(lds_read_tr(G::t_at(vp[0], mt)), lds_read_tr(G::t_at(vp[1], mt))), pb[ks],
                         o[mt]);
             }
-            store_token<BF, D, kLineStores<D, kOneHaloWgs<D, KS>>>(const_cast<short *>(image<short>(a.o, cur)) + lq.qr * a.o.sh + lq.qc * a.o.sw,
+            store_token<BF, D, kLineStores<D, KS, kOneHaloWgs<D, KS>>>(const_cast<short *>(image<short>(a.o, cur)) + lq.qr * a.o.sh + lq.qc * a.o.sw,
                                g, o, 1.f / sum, lq.live, dlim);
             if (lq.live && a.lse && g == 0)
                 a.lse[lq.tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
@@ -472,7 +476,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void b
                         dq[mt]);
             }
 
-            store_token<BF, D, kLineStores<D, G::WAVES>>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live, dlim);
+            store_token<BF, D, kLineStores<D, KS, G::WAVES>>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live, dlim);
             if (lq.live && g == 0) a.delta[lq.tok] = delta;
         }
 
@@ -604,7 +608,7 @@ __global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void bwd_dq2_mfma(BwdArg
                         cat(lds_read_tr(G::t_at(kp[0], mt)), lds_read_tr(G::t_at(kp[1], mt))), dsb[ks],
                         dq[mt]);
             }
-            store_token<BF, D, kLineStores<D, kOneHaloWgs<D, KS>>>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live, dlim);
+            store_token<BF, D, kLineStores<D, KS, kOneHaloWgs<D, KS>>>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live, dlim);
             if (lq.live && g == 0) a.delta[lq.tok] = delta;
         }
         if (!more) break;
@@ -816,8 +820,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         const int kr = cur.r0 + orow + (n >> 2), kc = cur.c0 + ocol + (n & 3);
         const int64_t goff = a.grad_at(cur.bb, cur.nn, kr, kc);
         if constexpr (SP == 1) {
-            store_token<BF, D, kLineStores<D, G::WAVES>>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, true, dlim);
-            store_token<BF, D, kLineStores<D, G::WAVES>>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, true, dlim);
+            store_token<BF, D, kLineStores<D, KS, G::WAVES>>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, true, dlim);
+            store_token<BF, D, kLineStores<D, KS, G::WAVES>>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, true, dlim);
             if (!more) break;
             load_keys(nxt);
             __syncthreads();
@@ -842,8 +846,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
                     dk[mt] += red[mt * 256];
                     dv[mt] += red[(G::DT + mt) * 256];
                 }
-                store_token<BF, D, kLineStores<D, G::WAVES>>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, true, dlim);
-                store_token<BF, D, kLineStores<D, G::WAVES>>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, true, dlim);
+                store_token<BF, D, kLineStores<D, KS, G::WAVES>>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, true, dlim);
+                store_token<BF, D, kLineStores<D, KS, G::WAVES>>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, true, dlim);
             }
             if (!more) break;
         }
@@ -1022,8 +1026,8 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
         const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
         auto store = [&]() __attribute__((always_inline)) {
             const int64_t goff = a.grad_at(cur.tl.bb, cur.tl.nn, kr, kc);
-            store_token<BF, D, kLineStores<D, fits<D, KS>() ? Geo<D, KS, 4, SP>::WAVES : 1>>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live, dlim);
-            store_token<BF, D, kLineStores<D, fits<D, KS>() ? Geo<D, KS, 4, SP>::WAVES : 1>>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live, dlim);
+            store_token<BF, D, kLineStores<D, KS, fits<D, KS>() ? Geo<D, KS, 4, SP>::WAVES : 1>>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live, dlim);
+            store_token<BF, D, kLineStores<D, KS, fits<D, KS>() ? Geo<D, KS, 4, SP>::WAVES : 1>>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live, dlim);
         };
         if constexpr (SP == 1) {
             if (cur.last) store();
