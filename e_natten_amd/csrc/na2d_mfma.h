@@ -124,9 +124,15 @@ __device__ __forceinline__ void store16(short *p, u32x4 v) {
 // extra HBM writes of the 64-byte runs (forward 73.1 -> 68.2 MB, dQ pass 73.5 -> 68.2, dK/dV
 // 148.6 -> 134.2, fused backward 222.8 -> 201.4 at B4 N4 128x128) and is used by the kernels
 // that run two workgroups per CU, which get 1-9% faster with it (forward 203 -> 194 us at
-// 256x256, dQ pass 61.8 -> 56.2, dK/dV 92.6 -> 86.7); the kernels with one workgroup per CU
-// get slower (fused backward 118 -> 139 us, dK/dV at k = 7 153 -> 165) and keep the 64-byte runs.
-template <bool BF, int D, bool LINES = false>
+// 256x256, dQ pass 61.8 -> 56.2, dK/dV 92.6 -> 86.7).  With predicated stores (`live`) the
+// kernels with one workgroup per CU get slower (fused backward 118 -> 139 us, dK/dV at k = 7
+// 153 -> 165): the branches that the predicates of the exchanged `live` flags put between the
+// stores cut the store sequence into blocks that nothing is scheduled across.  Where every
+// token exists (ALL: the fused backward, the inner tiles of the dK/dV pass) there are no
+// branches and the whole lines cost nothing (fused backward 123.8 -> 122.4 us with them on the
+// key side).
+// ALL: every lane's token exists (`live` is not looked at), so the stores are not predicated.
+template <bool BF, int D, bool LINES = false, bool ALL = false>
 __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *acc, float mul,
                                             bool live, int dlim = D) {
     constexpr int NP = D / 32;
@@ -187,10 +193,10 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
             // global-memory instructions: an address rebuilt from exchanged integers makes them flat)
             const uintptr_t own = reinterpret_cast<uintptr_t>(token);
             const uintptr_t nbr = (uintptr_t)xchg((unsigned)own) | ((uintptr_t)xchg((unsigned)(own >> 32)) << 32);
-            const bool nlive = xchg(live ? 1u : 0u) != 0;
+            const bool nlive = ALL || xchg(live ? 1u : 0u) != 0;
             short *other = reinterpret_cast<short *>(reinterpret_cast<char *>(token) + (ptrdiff_t)(nbr - own));
             short *tok_a = odd ? other : token, *tok_b = odd ? token : other;
-            const bool live_a = odd ? nlive : live, live_b = odd ? live : nlive;
+            const bool live_a = ALL || (odd ? nlive : live), live_b = ALL || (odd ? live : nlive);
             const int off = (odd ? 32 : 0) + g * 8;
             if (live_a) {
                 if (off < dlim) store16(tok_a + off, s0);

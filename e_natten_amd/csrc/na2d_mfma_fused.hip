@@ -418,7 +418,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                         cat(lds_read_tr(G::t_at(kp[0], mt)), lds_read_tr(G::t_at(kp[1], mt))), dsb[ks],
                         dq[mt]);
             }
-            store_token<BF, D>(static_cast<short *>(a.dq) + out_token() * D, g, dq, s.scale, true);
+            store_token<BF, D, false, true>(static_cast<short *>(a.dq) + out_token() * D, g, dq, s.scale, true);
         } else {
             auto issue = [&](int part) __attribute__((always_inline)) { issue_as(part, kKeySide); };
             // ---- key side: this lane's key is column n of every product
@@ -478,7 +478,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                                 cat(lds_read_tr(G::t_at(xt[0], mt)), lds_read_tr(G::t_at(xt[1], mt))), b[ks],
                                 acc[mt]);
                     }
-                    store_token<BF, D>(static_cast<short *>(out) + tok * D, g, acc, mul, true);
+                    store_token<BF, D, true, true>(static_cast<short *>(out) + tok * D, g, acc, mul, true);
                 };
                 second(lds_g, pb, a.dv, 1.f);
                 second(lds_q, dsb, a.dk, s.scale);
@@ -690,8 +690,8 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 issue(3);
                 issue(4);
                 const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + ky) * s.W + kx;
-                store_token<BF, D>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
-                store_token<BF, D>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
+                store_token<BF, D, true, true>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
+                store_token<BF, D, true, true>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
             }
         }
 

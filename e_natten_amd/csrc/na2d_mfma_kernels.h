@@ -47,6 +47,12 @@ namespace {
 // 61.4, dQ 67.8 -> 65.5, dK/dV 83.7 -> 76.1; B4 N4 256x256 k5 473 -> 427 per forward+backward;
 // k7 284 -> 282; no gain from k = 9 on (343 -> 347, 281.4 -> 280.9 at k13), where the kernels
 // do not wait for their stores, so it stops at 7 there.
+// The dK/dV pass's inner tiles have no token outside the image, so their whole-line stores
+// need no predicates (store_token's ALL), and without the branches that predicates put between
+// the stores they pay at one workgroup per CU as well: dK/dV pass d128 k7 157.5 -> 154.6 us, k5
+// 91.1 -> 88.7, d64 k5 82.1 -> 76.3, equal from k = 9 on.
+template <int D>
+constexpr bool kInnerLines = (D == 128 || D == 64) && !kNarrow;
 template <int D, int KS, int WGS>
 constexpr bool kLineStores = (D == 128 || (D == 64 && KS <= 7)) && !kNarrow && WGS >= 2;
 
@@ -820,8 +826,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
         const int kr = cur.r0 + orow + (n >> 2), kc = cur.c0 + ocol + (n & 3);
         const int64_t goff = a.grad_at(cur.bb, cur.nn, kr, kc);
         if constexpr (SP == 1) {
-            store_token<BF, D, kLineStores<D, KS, G::WAVES>>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, true, dlim);
-            store_token<BF, D, kLineStores<D, KS, G::WAVES>>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, true, dlim);
+            store_token<BF, D, kInnerLines<D>, true>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, true, dlim);
+            store_token<BF, D, kInnerLines<D>, true>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, true, dlim);
             if (!more) break;
             load_keys(nxt);
             __syncthreads();
@@ -846,8 +852,8 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
                     dk[mt] += red[mt * 256];
                     dv[mt] += red[(G::DT + mt) * 256];
                 }
-                store_token<BF, D, kLineStores<D, KS, G::WAVES>>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, true, dlim);
-                store_token<BF, D, kLineStores<D, KS, G::WAVES>>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, true, dlim);
+                store_token<BF, D, kInnerLines<D>, true>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, true, dlim);
+                store_token<BF, D, kInnerLines<D>, true>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, true, dlim);
             }
             if (!more) break;
         }
