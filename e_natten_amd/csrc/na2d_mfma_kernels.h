@@ -45,16 +45,11 @@ namespace {
 // on tensors of head_dim 128 or 64 itself (a token is then two aligned lines, or one).
 // Measured, us, without -> with: d = 128 see store_token; d = 64 B4 N8 128x128 k5 forward 65.4 ->
 // 61.4, dQ 67.8 -> 65.5, dK/dV 83.7 -> 76.1; B4 N4 256x256 k5 473 -> 427 per forward+backward;
-// k7 284 -> 282; no gain from k = 9 on (343 -> 347, 281.4 -> 280.9 at k13), where the kernels
-// do not wait for their stores, so it stops at 7 there.
-// The dK/dV pass's inner tiles have no token outside the image, so their whole-line stores
-// need no predicates (store_token's ALL), and without the branches that predicates put between
-// the stores they pay at one workgroup per CU as well: dK/dV pass d128 k7 157.5 -> 154.6 us, k5
-// 91.1 -> 88.7, d64 k5 82.1 -> 76.3, equal from k = 9 on.
-template <int D>
-constexpr bool kInnerLines = (D == 128 || D == 64) && !kNarrow;
+// k7 284 -> 282; from k = 9 on the times do not change (343 -> 347, 281.4 -> 280.9 at k13: the
+// kernels do not wait for their stores there), but the bytes do (dQ pass at d64 k13: 54.5 MB
+// written for 34.6), so it is used at every kernel size.
 template <int D, int KS, int WGS>
-constexpr bool kLineStores = (D == 128 || (D == 64 && KS <= 7)) && !kNarrow && WGS >= 2;
+constexpr bool kLineStores = (D == 128 || D == 64) && !kNarrow && WGS >= 2;
 
 // ------------------------------------------------------------------ forward
 // ROLL: walk down the columns of an image and keep the halo rows that consecutive
