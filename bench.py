@@ -366,8 +366,8 @@ def main():
         "path_frac": alg["path"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
     }
     path = kernel_path(D, ks, dtype)
-    if args.seq:   # the 1D matrix-core kernels: bf16 / f16, head_dim 32 / 64 / 128, kernel_size <= 49
-        path = "mfma" if path != "none" and args.dtype != "fp32" and D in (32, 64, 128) and 3 <= ks <= 49 \
+    if args.seq:   # the 1D matrix-core kernels: bf16 / f16, head dims that are multiples of 8 up to 128, kernel_size <= 49
+        path = "mfma" if path != "none" and args.dtype != "fp32" and D % 8 == 0 and 8 <= D <= 128 and 3 <= ks <= 49 \
             else "simt"
     if path == "mfma" and args.dtype in MFMA_PEAK_TF and not args.simt:
         # useful FLOPs against the matrix-core peak of the dtype the kernels compute in

@@ -17,7 +17,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libenatten.so")
 TORCH_LIB = os.path.join(HERE, "libenatten_torch.so")
 SOURCES = ["na2d_mfma.hip", "na2d_mfma_narrow.hip", "enatten_capi.hip", "enatten_prof.cpp", "na2d_simt.hip",
-           "na2d_f64.hip", "na2d_mfma_fused.hip", "na2d_mfma_onepass.hip", "na2d_mfma_f32.hip", "na1d_mfma.hip"]
+           "na2d_f64.hip", "na2d_mfma_fused.hip", "na2d_mfma_onepass.hip", "na2d_mfma_f32.hip", "na1d_mfma.hip", "na1d_mfma_narrow.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -139,6 +139,8 @@ int launch_bwd_mfma_narrow(const BwdArgs &a, int dtype, int path, hipStream_t st
 bool mfma1d_supported(int D, int ks, int dtype);
 int launch_fwd1d_mfma(const FwdArgs &a, int dtype, hipStream_t st);
 int launch_bwd1d_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st);
+int launch_fwd1d_mfma_narrow(const FwdArgs &a, int dtype, hipStream_t st);
+int launch_bwd1d_mfma_narrow(const BwdArgs &a, int dtype, int path, hipStream_t st);
 // fused backward (dQ, dK, dV of every tile from one staging), where built
 bool fused_bwd_supported(const BwdArgs &a);
 int launch_bwd_fused(const BwdArgs &a, bool bf16, const TileSet &ts, int64_t ntiles,

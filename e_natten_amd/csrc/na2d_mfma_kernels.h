@@ -48,6 +48,12 @@ namespace {
 // k7 284 -> 282; from k = 9 on the times do not change (343 -> 347, 281.4 -> 280.9 at k13: the
 // kernels do not wait for their stores there), but the bytes do (dQ pass at d64 k13: 54.5 MB
 // written for 34.6), so it is used at every kernel size.
+// The dK/dV pass's inner tiles have no token outside the image, so their whole-line stores
+// need no predicates (store_token's ALL), and without the branches that predicates put between
+// the stores they pay at one workgroup per CU as well: dK/dV pass d128 k7 157.5 -> 154.6 us, k5
+// 91.1 -> 88.7, d64 k5 82.1 -> 76.3, equal from k = 9 on.
+template <int D>
+constexpr bool kInnerLines = (D == 128 || D == 64) && !kNarrow;
 template <int D, int KS, int WGS>
 constexpr bool kLineStores = (D == 128 || D == 64) && !kNarrow && WGS >= 2;
 

@@ -83,6 +83,55 @@ def test_shapes_1d(shape, ks, dtype, path):
     _run(shape, dtype, ks, seed=2)
 
 
+@pytest.mark.parametrize("D,ks,T,dtype", [
+    (8, 3, 70, torch.bfloat16), (16, 7, 200, torch.bfloat16), (24, 13, 129, torch.float16),
+    (40, 5, 64, torch.bfloat16), (48, 33, 300, torch.bfloat16), (56, 17, 65, torch.bfloat16),
+    (72, 7, 500, torch.float16), (96, 19, 150, torch.bfloat16), (96, 49, 260, torch.bfloat16),
+    (120, 3, 33, torch.bfloat16), (104, 25, 400, torch.bfloat16),
+])
+def test_head_dims_between_the_built_ones_1d(D, ks, T, dtype, path, _lib):
+    """Head dims that are multiples of 8 run on the 1D matrix-core kernels of the next of 32, 64,
+    128.  Through the C ABI, every tensor a [.., D] view of a buffer with 8 more channels per
+    position (NaN beside the inputs, a marker beside the outputs): results against the oracle,
+    and no guard channel read or written."""
+    from e_natten_amd import _lib as L
+    B, N = 2, 3
+    shape = (B, N, T, D)
+    code = {torch.bfloat16: L.BF16, torch.float16: L.F16}[dtype]
+    g = torch.Generator().manual_seed(70 + D)
+    q, k, v, d_o = (torch.randn(shape, generator=g).to(dtype) for _ in range(4))
+    print("case narrow head dim 1d", shape, dtype, "k=%d" % ks, path, flush=True)
+    ref = O1.natten1d_explicit(q, k, v, d_o, ks, 1.0)
+    dev = torch.device("cuda:0")
+
+    def guarded(t=None):
+        buf = torch.full(shape[:-1] + (D + 8,), float("nan") if t is not None else 512.0, dtype=dtype, device=dev)
+        if t is not None:
+            buf[..., :D].copy_(t.to(dev))
+        return buf, buf[..., :D]
+
+    (_, qv), (_, kv), (_, vv), (_, gv) = (guarded(t) for t in (q, k, v, d_o))
+    (ob, ov), (dqb, dqv), (dkb, dkv), (dvb, dvv) = (guarded() for _ in range(4))
+    lse = torch.empty((B, N, T), dtype=torch.float32, device=dev)
+    ws = torch.empty(_lib.enatten1d_bwd_workspace_bytes(B, N, T), dtype=torch.uint8, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    sq, sk, sv, sg, so, sgr = (L.strides3(t) for t in (qv, kv, vv, gv, ov, dqv))
+    rc = _lib.enatten1d_fwd(qv.data_ptr(), kv.data_ptr(), vv.data_ptr(), ov.data_ptr(), lse.data_ptr(),
+                            B, N, T, D, ks, code, sq, sk, sv, so, 1.0, st)
+    assert rc == 0, L.last_error()
+    rc = _lib.enatten1d_bwd_into(qv.data_ptr(), kv.data_ptr(), vv.data_ptr(), ov.data_ptr(), gv.data_ptr(),
+                                 lse.data_ptr(), dqv.data_ptr(), dkv.data_ptr(), dvv.data_ptr(), ws.data_ptr(),
+                                 B, N, T, D, ks, code, sq, sk, sv, so, sg, sgr, 1.0, st)
+    assert rc == 0, L.last_error()
+    torch.cuda.synchronize()
+    for name, buf in (("O", ob), ("dQ", dqb), ("dK", dkb), ("dV", dvb)):
+        assert (buf[..., D:].float() == 512.0).all(), "%s: a guard channel was written" % name
+    for name, x, r in zip(("O", "dQ", "dK", "dV"), (ov, dqv, dkv, dvv), (ref[0], ref[2], ref[3], ref[4])):
+        x = x.float().cpu()
+        assert torch.isfinite(x).all(), name
+        assert O.rel_err(x, r) <= BF16_REL, (name, O.rel_err(x, r))
+
+
 def test_scale_and_c_oracle_1d():
     got, ref = _run((2, 2, 100, 64), torch.float32, 5, seed=3, scale=0.125)
     g = torch.Generator().manual_seed(3)
