@@ -216,20 +216,20 @@ constexpr bool kOneHaloFits = Geo<D, KS>::ROWS * Geo<D, KS>::PITCH * 2 + 1024 <=
 // flight, V over K behind a barrier, then O^T = V^T P^T while the next tile's K rows are in
 // flight.  Two workgroups per CU (one at kernel_size 11 and 13), four barriers per tile; 8x8
 // tiles, no column walk.
-template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void fwd2_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles) {
-    using G = Geo<D, KS>;
+template <bool BF, int D, int KS, int NW = 4>
+__global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS> : 1)) void fwd2_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles) {
+    using G = Geo<D, KS, NW>;
     __shared__ __attribute__((aligned(16))) short lds_x[G::ROWS * G::PITCH];
     const Shape &s = a.s;
     const int dlim = kNarrow ? s.D : D;  // head dim of the tensors: D, or less in the build for narrow dims
     Sched sc = make_sched(ntiles, blockIdx.x, gridDim.x);
     if (sc.t >= sc.t_end) return;
-    zero_row<D, KS>(lds_x, dlim);
+    zero_row<D, KS, NW>(lds_x, dlim);
 
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
-    const HaloPlan<D, KS> plan = make_plan<D, KS>(dlim);
-    HaloRegs<D, KS> st;
+    const HaloPlan<D, KS, NW> plan = make_plan<D, KS, NW>(dlim);
+    HaloRegs<D, KS, NW> st;
     s16x8 qnext[G::DS];
     auto fetch_rows = [&](const View &vw, const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
         halo_fetch<D, KS>(st, plan, image<short>(vw, tl), vw.sh, vw.sw, lq.hr0, lq.hc0, s.H, s.W);
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void fwd2_mfma(FwdArgs a
     auto fetch_q = [&](const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
         load_row_chunks(qnext, image<short>(a.q, tl) + lq.qr * a.q.sh + lq.qc * a.q.sw, g, dlim);
     };
-    Tile cur = tile_of(sc.t, tiles_r, tiles_c, s.N);
+    Tile cur = tile_of(sc.t, tiles_r, tiles_c, s.N, G::TH);
     LaneQ lq = lane_query<KS>(cur, s, wave, n);
     fetch_rows(a.k, cur, lq);
     fetch_q(cur, lq);
@@ -288,7 +288,7 @@ __global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void fwd2_mfma(FwdArgs a
         Tile nxt = cur;
         LaneQ lqn = lq;
         if (more) {
-            nxt = tile_of(tn, tiles_r, tiles_c, s.N);
+            nxt = tile_of(tn, tiles_r, tiles_c, s.N, G::TH);
             lqn = lane_query<KS>(nxt, s, wave, n);
             fetch_rows(a.k, nxt, lqn);
             fetch_q(nxt, lqn);
@@ -309,7 +309,7 @@ __global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void fwd2_mfma(FwdArgs a
                         cat(lds_read_tr(G::t_at(vp[0], mt)), lds_read_tr(G::t_at(vp[1], mt))), pb[ks],
                         o[mt]);
             }
-            store_token<BF, D, kLineStores<D, KS, kOneHaloWgs<D, KS>>>(const_cast<short *>(image<short>(a.o, cur)) + lq.qr * a.o.sh + lq.qc * a.o.sw,
+            store_token<BF, D, kLineStores<D, KS, (NW == 4 ? kOneHaloWgs<D, KS> : 1)>>(const_cast<short *>(image<short>(a.o, cur)) + lq.qr * a.o.sh + lq.qc * a.o.sw,
                                g, o, 1.f / sum, lq.live, dlim);
             if (lq.live && a.lse && g == 0)
                 a.lse[lq.tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
@@ -504,20 +504,20 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void b
 //   phase 2  K rows in LDS: P from the saved log-sum-exp, delta, dS, dQ^T = K^T dS^T;
 //            the next tile's V rows are in flight meanwhile.
 // Four barriers per tile instead of two; 8x8 tiles, no column walk.
-template <bool BF, int D, int KS>
-__global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void bwd_dq2_mfma(BwdArgs a, TileSet ts, int ntiles) {
-    using G = Geo<D, KS>;
+template <bool BF, int D, int KS, int NW = 4>
+__global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS> : 1)) void bwd_dq2_mfma(BwdArgs a, TileSet ts, int ntiles) {
+    using G = Geo<D, KS, NW>;
     __shared__ __attribute__((aligned(16))) short lds_x[G::ROWS * G::PITCH];
     const Shape &s = a.s;
     const int dlim = kNarrow ? s.D : D;  // head dim of the tensors: D, or less in the build for narrow dims
     Sched sc = make_sched(ntiles, blockIdx.x, gridDim.x);
     if (sc.t >= sc.t_end) return;
-    zero_row<D, KS>(lds_x, dlim);  // (a commit only writes the halo's own rows)
+    zero_row<D, KS, NW>(lds_x, dlim);  // (a commit only writes the halo's own rows)
 
     const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
-    const HaloPlan<D, KS> plan = make_plan<D, KS>(dlim);
-    HaloRegs<D, KS> st;
+    const HaloPlan<D, KS, NW> plan = make_plan<D, KS, NW>(dlim);
+    HaloRegs<D, KS, NW> st;
     // This lane's dO row is loaded a phase ahead of phase 1, its q row and log-sum-exp a
     // phase ahead of phase 2: one spare set of row registers instead of two.
     s16x8 qreg[G::DS], gnext[G::DS];
@@ -533,7 +533,7 @@ __global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void bwd_dq2_mfma(BwdArg
         lse_cur = a.lse[lq.tok];
     };
 
-    Tile cur = tile_of(sc.t, ts.tiles_r, ts.tiles_c, s.N);
+    Tile cur = tile_of(sc.t, ts.tiles_r, ts.tiles_c, s.N, G::TH);
     LaneQ lq = lane_query<KS>(cur, s, wave, n);
     fetch_rows(a.v, cur, lq);
     fetch_do(cur, lq);
@@ -568,7 +568,7 @@ __global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void bwd_dq2_mfma(BwdArg
         Tile nxt = cur;
         LaneQ lqn = lq;
         if (more) {
-            nxt = tile_of(tn, ts.tiles_r, ts.tiles_c, s.N);
+            nxt = tile_of(tn, ts.tiles_r, ts.tiles_c, s.N, G::TH);
             lqn = lane_query<KS>(nxt, s, wave, n);
             fetch_rows(a.v, nxt, lqn);
             fetch_do(nxt, lqn);
@@ -615,7 +615,7 @@ __global__ __launch_bounds__(256, (kOneHaloWgs<D, KS>)) void bwd_dq2_mfma(BwdArg
                         cat(lds_read_tr(G::t_at(kp[0], mt)), lds_read_tr(G::t_at(kp[1], mt))), dsb[ks],
                         dq[mt]);
             }
-            store_token<BF, D, kLineStores<D, KS, kOneHaloWgs<D, KS>>>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live, dlim);
+            store_token<BF, D, kLineStores<D, KS, (NW == 4 ? kOneHaloWgs<D, KS> : 1)>>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live, dlim);
             if (lq.live && g == 0) a.delta[lq.tok] = delta;
         }
         if (!more) break;
@@ -1184,6 +1184,17 @@ constexpr bool kDq2Built = (D == 64 || D == 128) && Geo<D, KS>::WAVES == 1 && !k
 // B1 N4 28.0 -> 22.4, B4 N4 106.6 -> 68.5.  With fewer tiles fwd_mfma's single workgroup
 // per CU is faster (B2 N2 64x64: 9.3 us against 9.9).  At head_dim 64 (kernel_size 11, 13)
 // the 16x8 tiles of fwd_mfma are faster (57.8 us against 59.3, 61.6 against 69.5).
+// 16x8 tiles with eight waves for the one-halo kernels where an 8x8 tile's halo leaves LDS for one
+// workgroup of four waves per CU (head_dim 128, kernel_size 11 and 13) and the taller halo still
+// fits (128 and 153 KB): two waves per SIMD instead of one, and a quarter less halo per pixel.
+// B4 N4 128x128, us, 8x8 -> 16x8: forward k13 137.8 -> 104.5 (B8 N8: 526 -> 385), k11 143.4 -> 130.4;
+// dQ pass k13 179.7 -> 167.7 (B8 N8: 736 -> 642), k11 185.2 -> 190.4 (it spills 36 registers
+// there), so the dQ pass takes the tall tiles at kernel_size 13 only.
+template <int D, int KS>
+constexpr bool kFwd2TallBuilt = D == 128 && kOneHaloWgs<D, KS> == 1 && kOneHaloFits<D, KS> &&
+                                (size_t)Geo<D, KS, 8>::ROWS * Geo<D, KS, 8>::PITCH * 2 + 1024 <= 160 * 1024;
+template <int D, int KS>
+constexpr bool kDq2TallBuilt = kFwd2TallBuilt<D, KS> && KS >= 13;
 template <int D, int KS>
 constexpr bool kFwd2Built = D == 128 && Geo<D, KS>::WAVES == 1 && kOneHaloFits<D, KS>;
 // Built at all: two halos fit, or the one-halo kernels serve the forward and the dQ pass and
@@ -1209,6 +1220,18 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
                 ProfScope prof(ENATTEN_KERNEL_FWD, "fwd_mfma", st);
                 hipLaunchKernelGGL((fwd_mfma<BF, D, KS, false, 8>), dim3(grid), dim3(G8::NT), 0, st, a,
                                    tall_r, tiles_c, (int)nb8, Runs{0, 0});
+                return check_launch("enatten2d_fwd");
+            }
+        }
+        if constexpr (kFwd2TallBuilt<D, KS>) {
+            using G8 = Geo<D, KS, 8>;
+            const int tall_r = (a.s.H + G8::TH - 1) / G8::TH;
+            const int64_t nb8 = (int64_t)a.s.B * a.s.N * tall_r * tiles_c;
+            if (nb8 >= 256) {  // a tile for every CU
+                const int grid = persistent_grid<fwd2_mfma<BF, D, KS, 8>>(nb8, G8::NT);
+                ProfScope prof(ENATTEN_KERNEL_FWD, "fwd2_mfma", st);
+                hipLaunchKernelGGL((fwd2_mfma<BF, D, KS, 8>), dim3(grid), dim3(G8::NT), 0, st, a, tall_r,
+                                   tiles_c, (int)nb8);
                 return check_launch("enatten2d_fwd");
             }
         }
@@ -1280,11 +1303,26 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         }
 
         bool dq_done = false;
+        if constexpr (kDq2TallBuilt<D, KS>) {
+            using G8 = Geo<D, KS, 8>;
+            TileSet tall = ts;  // only the tile counts are used by this pass
+            tall.tiles_r = (a.s.H + G8::TH - 1) / G8::TH;
+            const int64_t nb8 = slabs * tall.tiles_r * tiles_c;
+            if (nb8 >= 256) {
+                const int grid = persistent_grid<bwd_dq2_mfma<BF, D, KS, 8>>(nb8, G8::NT);
+                ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq2_mfma", st);
+                hipLaunchKernelGGL((bwd_dq2_mfma<BF, D, KS, 8>), dim3(grid), dim3(G8::NT), 0, st, a, tall,
+                                   (int)nb8);
+                dq_done = true;
+            }
+        }
         if constexpr (kDq2Built<D, KS>) {
-            const int grid = persistent_grid<bwd_dq2_mfma<BF, D, KS>>(nb);
-            ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq2_mfma", st);
-            hipLaunchKernelGGL((bwd_dq2_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, ts, (int)nb);
-            dq_done = true;
+            if (!dq_done) {
+                const int grid = persistent_grid<bwd_dq2_mfma<BF, D, KS>>(nb);
+                ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq2_mfma", st);
+                hipLaunchKernelGGL((bwd_dq2_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, ts, (int)nb);
+                dq_done = true;
+            }
         } else if constexpr (kTallDqBuilt<D, KS>) {
             using G8 = Geo<D, KS, 8>;
             TileSet tall = ts;  // only the tile counts are used by this pass
