@@ -1193,8 +1193,11 @@ constexpr bool kDq2Built = (D == 64 || D == 128) && Geo<D, KS>::WAVES == 1 && !k
 template <int D, int KS>
 constexpr bool kFwd2TallBuilt = D == 128 && kOneHaloWgs<D, KS> == 1 && kOneHaloFits<D, KS> &&
                                 (size_t)Geo<D, KS, 8>::ROWS * Geo<D, KS, 8>::PITCH * 2 + 1024 <= 160 * 1024;
+// At head_dim 64 (kernel_size 11 and 13, where one halo of an 8x8 tile fits LDS twice) the one-halo dQ
+// pass takes the 16x8 tiles too: one workgroup of eight waves instead of two of four, a quarter less halo
+// per pixel.  B2 N8 128x128 k13 81.5 -> 76.2 us, B4 N8 256x256 626 -> 606, B4 N4 128x128 k11 77.1 -> 76.3.
 template <int D, int KS>
-constexpr bool kDq2TallBuilt = kFwd2TallBuilt<D, KS> && KS >= 13;
+constexpr bool kDq2TallBuilt = (kFwd2TallBuilt<D, KS> && KS >= 13) || (D == 64 && KS >= 11);
 template <int D, int KS>
 constexpr bool kFwd2Built = D == 128 && Geo<D, KS>::WAVES == 1 && kOneHaloFits<D, KS>;
 // Built at all: two halos fit, or the one-halo kernels serve the forward and the dQ pass and
