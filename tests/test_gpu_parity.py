@@ -143,6 +143,8 @@ def test_one_halo_in_lds_at_a_time(shape, ks, dtype, _lib):
     ((1, 2, 13, 13, 128), 13, BF),      # window = image
     ((1, 1, 11, 40, 128), 11, F16),
     ((1, 2, 16, 24, 128), 13, BF),      # every key within reach of a border
+    ((4, 8, 37, 45, 128), 13, BF),      # enough 16x8 tiles for the eight-wave forward and dQ pass, ragged
+    ((3, 8, 50, 23, 128), 11, F16),     # (kernel_size 11: the forward only)
 ])
 def test_largest_windows_at_head_dim_128(shape, ks, dtype, _lib):
     # head_dim 128 with kernel_size 11 and 13 (the reference's own test sweeps kernel sizes up to
@@ -208,6 +210,12 @@ def test_one_pass_backward_fp16_and_strided_inputs(_lib):
 
 def test_config4_large_window(path):
     _case((2, 8, 128, 128, 64), BF, 13, what="C4")
+
+
+@pytest.mark.parametrize("shape,ks,dtype", [((4, 8, 41, 38, 64), 13, BF), ((4, 8, 35, 50, 64), 11, F16)])
+def test_large_windows_at_head_dim_64_on_ragged_images(shape, ks, dtype, path):
+    # the 16x8 tiles of the forward and of the one-halo dQ pass with a last tile that overhangs the image
+    _case(shape, dtype, ks, seed=17, what="d64 large window, ragged")
 
 
 @pytest.mark.parametrize("heads,side", [(2, 112), (4, 56), (8, 28), (16, 14)])
