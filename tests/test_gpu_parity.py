@@ -543,7 +543,7 @@ def test_tensors_beyond_2_31_elements(dtype, _lib):
     # 66 x 16 images of 128 x 128 x 128: 2.2e9 elements per tensor, so the element offset of
     # the last images does not fit 31 bits and their byte offset not 32.  Inputs are drawn
     # on the GPU; images at both ends and in the middle are compared with a call on a copy
-    # of that image alone (which the other tests hold against the oracle).
+    # of that image alone, and the last image with the CPU oracle.
     from e_natten_amd import natten2d
     dev = torch.device("cuda:0")
     B, N, H, W, D = 66, 16, 128, 128, 128
@@ -564,6 +564,11 @@ def test_tensors_beyond_2_31_elements(dtype, _lib):
             err = (x - r).abs().max().item()
             bound = 1e-5 if dtype == F32 else 2 ** -7 * r.abs().max().item()
             assert err <= bound, "%s of image (%d, %d): %.3e > %.3e" % (name, b, n, err, bound)
+    # and the last image, the one farthest beyond 2^31 elements, against the CPU oracle itself
+    qc, kc, vc, gc = (t[B - 1:, N - 1:].detach().cpu() for t in (q, k, v, g))
+    ref = oracle_all(qc, kc, vc, gc, 5)
+    got = tuple(t[B - 1:, N - 1:].detach().cpu() for t in (o,) + grads)
+    assert_close(got, (ref[0], ref[2], ref[3], ref[4]), dtype, "last image of a tensor beyond 2^31 elements")
     del q, k, v, g, o, grads
     torch.cuda.empty_cache()
 
