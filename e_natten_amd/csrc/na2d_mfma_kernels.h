@@ -1293,12 +1293,14 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         // At these head dims the passes are bound by per-tile latency, not by HBM, so reading
         // the inputs once only pays where the two passes are at their worst: images that are
         // (nearly) all border tiles, which the dK/dV pass walks block by block and the one-pass
-        // kernel serves from its one staged block.  Measured, backward only, one pass vs two
-        // (us, bf16): B8 N16 14x14 d32 k7 20.4 vs 21.9; B8 N8 28x28 d32 k7 29.7 vs 33.8, k5 24.4 vs
-        // 27.4; B16 N8 16x16 d32 k3 12.2 vs 16.1; but B8 N4 40x40 d32 k7 27.9 vs 25.1 (9 of 25
-        // tiles inner), B8 N8 28x28 d64 k3 30.9 vs 26.2 (4 of 16), B8 N2 112x112 d32 k7 66 vs 54,
-        // B4 N8 128x128 d32 k5 145 vs 87.  So it is the default where at most one tile in eight
-        // is an inner tile; ENATTEN_PATH_MFMA_FUSED forces it wherever it is built.
+        // kernel serves from its one staged block.  Measured on a settled GPU, backward kernels,
+        // one pass vs two (us, bf16, head_dim 32, kernel_size 7): B8 N16 14x14 17.2 vs 13.2;
+        // B8 N8 28x28 24.9 vs 24.8; B8 N4 40x40 22.0 vs 16.1 (9 of 25 tiles inner); B8 N4 56x56
+        // 32.6 vs 26.4; B8 N2 112x112 51.4 vs 42.8.  The whole step replayed as a graph, where
+        // one launch less counts: 14x14 30.3 vs 29.0, 28x28 39.2 vs 40.7, 40x40 37.8 vs 32.9,
+        // 56x56 52.7 vs 49.0.  So it is the default only where at most one tile in eight is an
+        // inner tile (level with the two passes there, one launch less);
+        // ENATTEN_PATH_MFMA_FUSED forces it wherever it is built.
         if (path != ENATTEN_PATH_MFMA_SPLIT && onepass_bwd_supported(a) &&
             (path == ENATTEN_PATH_MFMA_FUSED || 8 * n_inner <= nb)) {
             const int rc = launch_bwd_onepass(a, BF, ts, nb, st);
