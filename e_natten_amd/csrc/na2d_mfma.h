@@ -66,25 +66,26 @@ __device__ __forceinline__ float col_sum(float x) {
     return x + __shfl_xor(x, 32, 64);
 }
 
-// dO . O over the 8 channels of one 16-byte chunk, in float32 FMAs.  The halves of
-// a dword are taken apart with integer operations: a bit_cast of a vector element
-// to a 2-vector of 16-bit floats makes this compiler read the chunk's first dword
-// four times (seen in the generated code, and in wrong results).
-template <bool BF>
-__device__ __forceinline__ float half_of(uint32_t w, bool high) {
-    const uint32_t h = high ? w >> 16 : w & 0xffffu;
-    if constexpr (BF) return __uint_as_float(h << 16);
-    else return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
-}
+// dO . O over the 8 channels of one 16-byte chunk: four two-element dot products that
+// accumulate in float32 (v_dot2c_f32_bf16 / v_dot2c_f32_f16), one instruction per dword where
+// taking the halves apart and multiplying them took six.
 template <bool BF>
 __device__ __forceinline__ float dot8(u32x4 a, u32x4 b) {
-    float even = 0.f, odd = 0.f;
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    float acc = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        even = fmaf(half_of<BF>(a[j], false), half_of<BF>(b[j], false), even);
-        odd = fmaf(half_of<BF>(a[j], true), half_of<BF>(b[j], true), odd);
+        // (the dwords are taken out of the vectors as integers first: a bit_cast of a vector
+        // element to a 2-vector of 16-bit floats made this compiler read the chunk's first
+        // dword four times)
+        const uint32_t x = a[j], y = b[j];
+        if constexpr (BF)
+            acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, x), __builtin_bit_cast(bf16x2, y), acc, false);
+        else
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, x), __builtin_bit_cast(f16x2, y), acc, false);
     }
-    return even + odd;
+    return acc;
 }
 // sum over aligned groups of LANES (4, 8 or 16) consecutive lanes, in every lane
 template <int LANES>
