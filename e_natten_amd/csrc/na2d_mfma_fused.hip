@@ -73,7 +73,10 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
     __shared__ __attribute__((aligned(16))) short lds_g[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
-    __shared__ float2 lds_stat[G::ROWS];  // (log-sum-exp * log2(e), dO . O) per staged query
+    // (log-sum-exp * log2(e), scale * dO . O) per staged query.  dS is formed with the softmax
+    // scale in it, p * (scale * dP - scale * delta): one fused multiply-add where the difference
+    // was one subtraction, and dQ and dK leave their accumulators without 32 multiplications each.
+    __shared__ float2 lds_stat[G::ROWS];
     // per key-side wave, for a tile beside a border: LDS row | region row << 16 | region
     // column << 20 of each of its 64 query numbers
     __shared__ int lds_qtab[4 * 64];
@@ -254,7 +257,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 *reinterpret_cast<u32x4 *>(lds_g + e) = gst.v[i];
                 *reinterpret_cast<u32x4 *>(lds_k + e) = kst.v[i];
                 *reinterpret_cast<u32x4 *>(lds_v + e) = vst.v[i];
-                if (ch8_of() == 0) lds_stat[row].y = d;
+                if (ch8_of() == 0) lds_stat[row].y = d * s.scale;
             }
         }
         if (stid < NR * G::HC) lds_stat[lds_row(stid / G::HC, stid % G::HC)].x = lse_st * kLog2e;
@@ -307,9 +310,19 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
             qst = fresh; gst = fresh; kst = fresh; vst = fresh; ost = fresh;
         }
         int round_n = deal_round;
-        const int tn = tile_after(sc.t, round_n);
-        const bool more = tn < sc.t_end;
-        const Tile nxt = more ? tile_of_cm(tn, ts.tiles_r, ts.tiles_c, s.N) : cur;
+        int tn;
+        bool more;
+        Tile nxt = cur;
+        if ((deal_ncols == 0 || sc.t + 1 < seg_end) && sc.t + 1 < sc.t_end && cur.r0 + 8 < s.H) {
+            // the usual step, to the tile below in the same column: no divisions
+            tn = sc.t + 1;
+            more = true;
+            nxt.r0 = cur.r0 + 8;
+        } else {
+            tn = tile_after(sc.t, round_n);
+            more = tn < sc.t_end;
+            if (more) nxt = tile_of_cm(tn, ts.tiles_r, ts.tiles_c, s.N);
+        }
         // the tile below in the same image: its block shares k-1 rows with this one
         const bool below = more && nxt.bb == cur.bb && nxt.nn == cur.nn && nxt.c0 == cur.c0 &&
                            nxt.r0 == cur.r0 + 8;
@@ -394,7 +407,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 }
             }
             const float2 mine = lds_stat[prow];
-            const float lse2 = mine.x, delta = mine.y;
+            const float lse2 = mine.x, delta_s = mine.y;
             s16x8 dsb[G::KSTEPS];
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
@@ -413,7 +426,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                     const bool ok = ((unsigned)(2 * mt + (g >> 1) - dr) < (unsigned)KS) &
                                     ((unsigned)(4 * (g & 1) + i - dc) < (unsigned)KS);
                     const float p = __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - lse2 : -INFINITY);
-                    dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - delta));
+                    dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * fmaf(cp[i], s.scale, -delta_s));
                 }
             }
             issue(4);
@@ -432,7 +445,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                         cat(lds_read_tr(G::t_at(kp[0], mt)), lds_read_tr(G::t_at(kp[1], mt))), dsb[ks],
                         dq[mt]);
             }
-            store_token<BF, D, false, true>(static_cast<short *>(a.dq) + out_token() * D, g, dq, s.scale, true);
+            store_token<BF, D, false, true>(static_cast<short *>(a.dq) + out_token() * D, g, dq, 1.f, true);
             finish_as(kQuerySide);
         } else {
             auto issue = [&](int part) __attribute__((always_inline)) { issue_as(part, kKeySide); };
@@ -472,7 +485,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                             const float2 st = stat(mt, i);
                             const float p = __builtin_amdgcn_exp2f(keep_or_ninf(cs[i] * sc2 - st.x, ok_fn(mt, i)));
                             pb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p);
-                            dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
+                            dsb[mt >> 1][(mt & 1) * 4 + i] = cvt16<BF>(p * fmaf(cp[i], s.scale, -st.y));
                         }
                     }
                 }
@@ -496,7 +509,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                     store_token<BF, D, true, true>(static_cast<short *>(out) + tok * D, g, acc, mul, true);
                 };
                 second(lds_g, pb, a.dv, 1.f);
-                second(lds_q, dsb, a.dk, s.scale);
+                second(lds_q, dsb, a.dk, 1.f);
             };
             const bool edge_r = tr == 0 || tr == ts.tiles_r - 1, edge_c = tc == 0 || tc == ts.tiles_c - 1;
             if (inner) {
@@ -683,7 +696,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                             const float2 st = lds_stat[row_of(tk)];
                             const float p = __builtin_amdgcn_exp2f(keep_or_ninf(cs[i] * sc2 - st.x, ok_of(tk)));
                             pb[m2 * 4 + i] = cvt16<BF>(p);
-                            dsb[m2 * 4 + i] = cvt16<BF>(p * (cp[i] - st.y));
+                            dsb[m2 * 4 + i] = cvt16<BF>(p * fmaf(cp[i], s.scale, -st.y));
                         }
                     }
                     typename G::TRow qt[2], gt[2];
@@ -705,7 +718,7 @@ __global__ __launch_bounds__(512) void bwd_fused_mfma(BwdArgs a, TileSet ts, int
                 issue(3);
                 issue(4);
                 const int64_t tok = (((int64_t)cur.bb * s.N + cur.nn) * s.H + ky) * s.W + kx;
-                store_token<BF, D, true, true>(static_cast<short *>(a.dk) + tok * D, g, dk, s.scale, true);
+                store_token<BF, D, true, true>(static_cast<short *>(a.dk) + tok * D, g, dk, 1.f, true);
                 store_token<BF, D, true, true>(static_cast<short *>(a.dv) + tok * D, g, dv, 1.f, true);
             }
             finish_as(kKeySide);
