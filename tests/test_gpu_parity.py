@@ -260,6 +260,10 @@ def test_edge_shapes(shape, ks, dtype, path):
 def test_scale_argument(path):
     _case((1, 2, 16, 20, 64), BF, 5, scale=0.125, small=True, what="scale")
     _case((1, 2, 12, 12, 16), F32, 3, scale=0.25, small=True, what="scale")
+    # the one-kernel backward of head_dim 128, kernel_size 5 and the one-pass backward of
+    # head_dim 32 form dS with the scale in it; a scale that is no power of two
+    _case((1, 2, 24, 32, 128), BF, 5, scale=0.3, what="scale, fused backward")
+    _case((2, 2, 16, 24, 32), BF, 7, scale=0.17, what="scale, one-pass backward")
 
 
 def test_strided_qkv_views(path):
