@@ -207,7 +207,7 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
                 if (off < dlim) store16(tok_b + off, s2);
                 if (off + 64 < dlim) store16(tok_b + off + 64, s3);
             }
-        } else if (live) {
+        } else if (ALL || live) {
 #pragma unroll
             for (int j = 0; j < NP; j++)
                 if (j * (D / 4) + g * 8 < dlim) store16(token + j * (D / 4) + g * 8, p[j]);
@@ -229,14 +229,14 @@ __device__ __forceinline__ void store_token(short *token, int g, const f32x4 *ac
         }
         const uintptr_t own = reinterpret_cast<uintptr_t>(token);
         const uintptr_t nbr = (uintptr_t)xchg((unsigned)own) | ((uintptr_t)xchg((unsigned)(own >> 32)) << 32);
-        const bool nlive = xchg(live ? 1u : 0u) != 0;
+        const bool nlive = ALL || xchg(live ? 1u : 0u) != 0;
         short *other = reinterpret_cast<short *>(reinterpret_cast<char *>(token) + (ptrdiff_t)(nbr - own));
         const int off = g * 16 + (odd ? 8 : 0);
-        if ((odd ? nlive : live) && off < dlim) store16((odd ? other : token) + off, s0);
-        if ((odd ? live : nlive) && off < dlim) store16((odd ? token : other) + off, s1);
+        if ((ALL || (odd ? nlive : live)) && off < dlim) store16((odd ? other : token) + off, s0);
+        if ((ALL || (odd ? live : nlive)) && off < dlim) store16((odd ? token : other) + off, s1);
     } else {
         // D = 32: the four lanes of a token already cover its 64 bytes.
-        if (live) {
+        if (ALL || live) {
 #pragma unroll
             for (int j = 0; j < NP; j++)
                 if (g * (D / 4) + j * 8 < dlim) store16(token + g * (D / 4) + j * 8, p[j]);
