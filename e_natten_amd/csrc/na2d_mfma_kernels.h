@@ -80,9 +80,8 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
     zero_row<D, KS, NW>(lds_k, dlim);
     zero_row<D, KS, NW>(lds_v, dlim);
 
-    // (the wave number through readfirstlane: the compiler then knows that it is uniform, and
-    // `wave_on` below is a scalar branch with two exclusive sides)
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const int wave = FULL ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : threadIdx.x >> 6;
+    const int l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
 
     // registers that carry the next tile while the current one is computed
@@ -109,10 +108,10 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
     int y0 = lq.hr0, nr = G::HR;
     prefetch(cur, lq, y0, nr);
     s16x8 qreg[G::DS];
-    // The staged rows go to LDS at the END of a tile's pass through the loop, after its stores,
-    // not at the top of the next: there the compiler has to merge the first pass (where these
-    // loads are the youngest memory operations) with the later ones, and waits for everything
-    // outstanding, the tile's own stores included.
+    // FULL: the staged rows go to LDS at the END of a tile's pass through the loop, after its
+    // stores, not at the top of the next: there the compiler has to merge the first pass (where
+    // these loads are the youngest memory operations) with the later ones, and waits for
+    // everything outstanding, the tile's own stores included.
     auto commit = [&]() __attribute__((always_inline)) {
         if constexpr (ROLL) {
             halo_commit_rows<D, KS>(lds_k, plan, kst, y0, nr);
@@ -124,8 +123,9 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) qreg[ds] = qnext[ds];
     };
-    commit();
+    if constexpr (FULL) commit();
     for (;;) {
+        if constexpr (!FULL) commit();
         __syncthreads();
 
         const int tn = sched_peek(sc);
@@ -144,7 +144,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
         } else {
             // (the last tile of the walk: nothing is loaded, and the explicit wait says so to
             // the compiler, which does not know that this path leaves the loop below)
-            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+            if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         }
         const int rot = ROLL ? lq.hr0 % G::HR : 0;
         auto trow = [&](int tile, int x) __attribute__((always_inline)) {
@@ -210,11 +210,11 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (Geo<D, KS, NW>::WAVES)) void
         }
 
         if (!more) {
-            __builtin_amdgcn_s_waitcnt(0x0F70);  // (as above: this path shares its last block with the other)
+            if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // (as above: this path shares its last block with the other)
             break;
         }
         __syncthreads();  // every wave is done with this tile's LDS
-        commit();
+        if constexpr (FULL) commit();
         cur = nxt;
         lq = lqn;
         sched_advance(sc, tn);
@@ -241,7 +241,8 @@ constexpr bool kOneHaloFits = Geo<D, KS>::ROWS * Geo<D, KS>::PITCH * 2 + 1024 <=
 // flight, V over K behind a barrier, then O^T = V^T P^T while the next tile's K rows are in
 // flight.  Two workgroups per CU (one at kernel_size 11 and 13), four barriers per tile; 8x8
 // tiles, no column walk.
-template <bool BF, int D, int KS, int NW = 4>
+// FULL: as in fwd_mfma.
+template <bool BF, int D, int KS, int NW = 4, bool FULL = false>
 __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS> : 1)) void fwd2_mfma(FwdArgs a, int tiles_r, int tiles_c, int ntiles) {
     using G = Geo<D, KS, NW>;
     __shared__ __attribute__((aligned(16))) short lds_x[G::ROWS * G::PITCH];
@@ -251,7 +252,8 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS, NW>(lds_x, dlim);
 
-    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const int wave = FULL ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : threadIdx.x >> 6;
+    const int l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
     const HaloPlan<D, KS, NW> plan = make_plan<D, KS, NW>(dlim);
     HaloRegs<D, KS, NW> st;
@@ -266,17 +268,23 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
     LaneQ lq = lane_query<KS>(cur, s, wave, n);
     fetch_rows(a.k, cur, lq);
     fetch_q(cur, lq);
-    for (;;) {
-        halo_commit<D, KS>(lds_x, plan, st);  // K
-        s16x8 qreg[G::DS];
+    s16x8 qreg[G::DS];
+    // (K rows and the query row at the end of a tile's pass through the loop, after its stores:
+    // see fwd_mfma)
+    auto commit_k = [&]() __attribute__((always_inline)) {
+        halo_commit<D, KS>(lds_x, plan, st);
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) qreg[ds] = qnext[ds];
+    };
+    if constexpr (FULL) commit_k();
+    for (;;) {
+        if constexpr (!FULL) commit_k();
         __syncthreads();
         fetch_rows(a.v, cur, lq);
         auto trow = [&](int tile, int x) __attribute__((always_inline)) { return G::token_row(tile, x, lq.orow, lq.ocol); };
         s16x8 pb[G::KSTEPS];
         float mx = -INFINITY, sum = 0.f;
-        if (lq.wave_on) {
+        if (FULL || lq.wave_on) {
             f32x4 acc[G::MT];
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
@@ -317,8 +325,10 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
             lqn = lane_query<KS>(nxt, s, wave, n);
             fetch_rows(a.k, nxt, lqn);
             fetch_q(nxt, lqn);
+        } else {
+            if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the last tile, nothing is loaded (see fwd_mfma)
         }
-        if (lq.wave_on) {
+        if (FULL || lq.wave_on) {
             f32x4 o[G::DT];
 #pragma unroll
             for (int mt = 0; mt < G::DT; mt++) o[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -334,13 +344,17 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
                         cat(lds_read_tr(G::t_at(vp[0], mt)), lds_read_tr(G::t_at(vp[1], mt))), pb[ks],
                         o[mt]);
             }
-            store_token<BF, D, kLineStores<D, KS, (NW == 4 ? kOneHaloWgs<D, KS> : 1)>>(const_cast<short *>(image<short>(a.o, cur)) + lq.qr * a.o.sh + lq.qc * a.o.sw,
+            store_token<BF, D, kLineStores<D, KS, (NW == 4 ? kOneHaloWgs<D, KS> : 1)>, FULL>(const_cast<short *>(image<short>(a.o, cur)) + lq.qr * a.o.sh + lq.qc * a.o.sw,
                                g, o, 1.f / sum, lq.live, dlim);
-            if (lq.live && a.lse && g == 0)
+            if (a.lse && (FULL || (lq.live && g == 0)))
                 a.lse[lq.tok] = (mx + __builtin_amdgcn_logf(sum)) * kLn2;
         }
-        if (!more) break;
+        if (!more) {
+            if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), see fwd_mfma
+            break;
+        }
         __syncthreads();  // every wave has read V
+        if constexpr (FULL) commit_k();
         cur = nxt;
         lq = lqn;
         sched_advance(sc, tn);
@@ -377,7 +391,8 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void b
     zero_row<D, KS, NW>(lds_k, dlim);
     zero_row<D, KS, NW>(lds_v, dlim);
 
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const int wave = FULL ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : threadIdx.x >> 6;
+    const int l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
     auto pick = [&](int t) __attribute__((always_inline)) {
         if constexpr (FRAME) return frame_tile(t, ts, s.N);
@@ -425,8 +440,9 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void b
         }
         lse2 = lse_next * kLog2e;
     };
-    commit();
+    if constexpr (FULL) commit();
     for (;;) {
+        if constexpr (!FULL) commit();
         __syncthreads();
 
         const int tn = sched_peek(sc);
@@ -443,7 +459,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void b
             nr = below ? lqn.hr0 - lq.hr0 : G::HR;
             prefetch(nxt, lqn, y0, nr);
         } else {
-            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the last tile, nothing is loaded (see fwd_mfma)
+            if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the last tile, nothing is loaded (see fwd_mfma)
         }
         const int rot = ROLL ? lq.hr0 % G::HR : 0;
         auto trow = [&](int tile, int x) __attribute__((always_inline)) {
@@ -522,11 +538,11 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void b
         }
 
         if (!more) {
-            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), see fwd_mfma
+            if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), see fwd_mfma
             break;
         }
         __syncthreads();
-        commit();
+        if constexpr (FULL) commit();
         cur = nxt;
         lq = lqn;
         sched_advance(sc, tn);
@@ -542,7 +558,8 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void b
 //   phase 2  K rows in LDS: P from the saved log-sum-exp, delta, dS, dQ^T = K^T dS^T;
 //            the next tile's V rows are in flight meanwhile.
 // Four barriers per tile instead of two; 8x8 tiles, no column walk.
-template <bool BF, int D, int KS, int NW = 4>
+// FULL: as in fwd_mfma.
+template <bool BF, int D, int KS, int NW = 4, bool FULL = false>
 __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS> : 1)) void bwd_dq2_mfma(BwdArgs a, TileSet ts, int ntiles) {
     using G = Geo<D, KS, NW>;
     __shared__ __attribute__((aligned(16))) short lds_x[G::ROWS * G::PITCH];
@@ -552,7 +569,8 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
     if (sc.t >= sc.t_end) return;
     zero_row<D, KS, NW>(lds_x, dlim);  // (a commit only writes the halo's own rows)
 
-    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const int wave = FULL ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : threadIdx.x >> 6;
+    const int l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
     const HaloPlan<D, KS, NW> plan = make_plan<D, KS, NW>(dlim);
     HaloRegs<D, KS, NW> st;
@@ -575,18 +593,24 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
     LaneQ lq = lane_query<KS>(cur, s, wave, n);
     fetch_rows(a.v, cur, lq);
     fetch_do(cur, lq);
-    for (;;) {
-        halo_commit<D, KS>(lds_x, plan, st);  // V
-        s16x8 greg[G::DS];
+    s16x8 greg[G::DS];
+    // (V rows and the dO row at the end of a tile's pass through the loop, after its stores:
+    // see fwd_mfma)
+    auto commit_v = [&]() __attribute__((always_inline)) {
+        halo_commit<D, KS>(lds_x, plan, st);
 #pragma unroll
         for (int ds = 0; ds < G::DS; ds++) greg[ds] = gnext[ds];
+    };
+    if constexpr (FULL) commit_v();
+    for (;;) {
+        if constexpr (!FULL) commit_v();
         __syncthreads();
         fetch_rows(a.k, cur, lq);
         fetch_q(cur, lq);
         auto trow = [&](int tile, int x) __attribute__((always_inline)) { return G::token_row(tile, x, lq.orow, lq.ocol); };
 
         f32x4 dp[G::MT];
-        if (lq.wave_on) {
+        if (FULL || lq.wave_on) {
 #pragma unroll
             for (int mt = 0; mt < G::MT; mt++) {
                 const typename G::ARow vp = G::a_row(lds_x, trow(mt, n), g);
@@ -610,9 +634,11 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
             lqn = lane_query<KS>(nxt, s, wave, n);
             fetch_rows(a.v, nxt, lqn);
             fetch_do(nxt, lqn);
+        } else {
+            if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the last tile, nothing is loaded (see fwd_mfma)
         }
         const float lse2 = lse_cur * kLog2e;
-        if (lq.wave_on) {
+        if (FULL || lq.wave_on) {
             s16x8 dsb[G::KSTEPS];
             float dpart = 0.f;
 #pragma unroll
@@ -653,11 +679,15 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
                         cat(lds_read_tr(G::t_at(kp[0], mt)), lds_read_tr(G::t_at(kp[1], mt))), dsb[ks],
                         dq[mt]);
             }
-            store_token<BF, D, kLineStores<D, KS, (NW == 4 ? kOneHaloWgs<D, KS> : 1)>>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live, dlim);
-            if (lq.live && g == 0) a.delta[lq.tok] = delta;
+            store_token<BF, D, kLineStores<D, KS, (NW == 4 ? kOneHaloWgs<D, KS> : 1)>, FULL>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live, dlim);
+            if (FULL || (lq.live && g == 0)) a.delta[lq.tok] = delta;
         }
-        if (!more) break;
+        if (!more) {
+            if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), see fwd_mfma
+            break;
+        }
         __syncthreads();  // every wave has read K
+        if constexpr (FULL) commit_v();
         cur = nxt;
         lq = lqn;
         sched_advance(sc, tn);
@@ -1275,8 +1305,12 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
             if (nb8 >= 256) {  // a tile for every CU
                 const int grid = persistent_grid<fwd2_mfma<BF, D, KS, 8>>(nb8, G8::NT);
                 ProfScope prof(ENATTEN_KERNEL_FWD, "fwd2_mfma", st);
-                hipLaunchKernelGGL((fwd2_mfma<BF, D, KS, 8>), dim3(grid), dim3(G8::NT), 0, st, a, tall_r,
-                                   tiles_c, (int)nb8);
+                if (!kNarrow && a.s.H % G8::TH == 0 && a.s.W % G8::TW == 0)
+                    hipLaunchKernelGGL((fwd2_mfma<BF, D, KS, 8, !kNarrow>), dim3(grid), dim3(G8::NT), 0, st, a,
+                                       tall_r, tiles_c, (int)nb8);
+                else
+                    hipLaunchKernelGGL((fwd2_mfma<BF, D, KS, 8>), dim3(grid), dim3(G8::NT), 0, st, a, tall_r,
+                                       tiles_c, (int)nb8);
                 return check_launch("enatten2d_fwd");
             }
         }
@@ -1284,8 +1318,12 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
             const int grid = persistent_grid<fwd2_mfma<BF, D, KS>>(nb);
             if (nb >= 2 * 256 || !fits<D, KS>()) {  // two workgroups for each of the 256 CUs
                 ProfScope prof(ENATTEN_KERNEL_FWD, "fwd2_mfma", st);
-                hipLaunchKernelGGL((fwd2_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
-                                   tiles_c, (int)nb);
+                if (!kNarrow && a.s.H % G::TH == 0 && a.s.W % G::TW == 0)
+                    hipLaunchKernelGGL((fwd2_mfma<BF, D, KS, 4, !kNarrow>), dim3(grid), dim3(256), 0, st, a,
+                                       tiles_r, tiles_c, (int)nb);
+                else
+                    hipLaunchKernelGGL((fwd2_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, tiles_r,
+                                       tiles_c, (int)nb);
                 return check_launch("enatten2d_fwd");
             }
         }
@@ -1314,6 +1352,13 @@ int fwd_launch(const FwdArgs &a, hipStream_t st) {
         return ENATTEN_EUNSUPPORTED;
     }
 }
+
+// Where the FULL form of bwd_dq2_mfma is used: at head_dim 128 it was measured faster with
+// kernel_size 7 and 11 (B4 N4 128x128: 76.7 -> 68.2 and 184.7 -> 173.2 us) and slower with 9
+// and 13 (82.4 -> 84.4, and 167.5 -> 214.7 with the 16x8 tiles: what those two spill moves
+// into their inner loops); at head_dim 64 faster (k11 76.2 -> 73.9, k13 76.2 -> 75.6).
+template <int D, int KS>
+constexpr bool kDq2Full = !kNarrow && (D != 128 || KS == 7 || KS == 11);
 
 template <bool BF, int D, int KS>
 int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
@@ -1367,8 +1412,12 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             if (nb8 >= 256) {
                 const int grid = persistent_grid<bwd_dq2_mfma<BF, D, KS, 8>>(nb8, G8::NT);
                 ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq2_mfma", st);
-                hipLaunchKernelGGL((bwd_dq2_mfma<BF, D, KS, 8>), dim3(grid), dim3(G8::NT), 0, st, a, tall,
-                                   (int)nb8);
+                if (kDq2Full<D, KS> && a.s.H % G8::TH == 0 && a.s.W % G8::TW == 0)
+                    hipLaunchKernelGGL((bwd_dq2_mfma<BF, D, KS, 8, kDq2Full<D, KS>>), dim3(grid), dim3(G8::NT), 0,
+                                       st, a, tall, (int)nb8);
+                else
+                    hipLaunchKernelGGL((bwd_dq2_mfma<BF, D, KS, 8>), dim3(grid), dim3(G8::NT), 0, st, a, tall,
+                                       (int)nb8);
                 dq_done = true;
             }
         }
@@ -1376,7 +1425,11 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             if (!dq_done) {
                 const int grid = persistent_grid<bwd_dq2_mfma<BF, D, KS>>(nb);
                 ProfScope prof(ENATTEN_KERNEL_BWD_DQ, "bwd_dq2_mfma", st);
-                hipLaunchKernelGGL((bwd_dq2_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, ts, (int)nb);
+                if (kDq2Full<D, KS> && a.s.H % G::TH == 0 && a.s.W % G::TW == 0)
+                    hipLaunchKernelGGL((bwd_dq2_mfma<BF, D, KS, 4, kDq2Full<D, KS>>), dim3(grid), dim3(256), 0, st,
+                                       a, ts, (int)nb);
+                else
+                    hipLaunchKernelGGL((bwd_dq2_mfma<BF, D, KS>), dim3(grid), dim3(256), 0, st, a, ts, (int)nb);
                 dq_done = true;
             }
         } else if constexpr (kTallDqBuilt<D, KS>) {
