@@ -481,7 +481,14 @@ __global__ __launch_bounds__(256, 2) void bwd1d_dkdv_mfma(BwdArgs a, int tiles_t
 // Workgroups per CU that the registers are budgeted for: what LDS admits, at most three.
 // (At head_dim 128 LDS holds one workgroup; a variant with eight waves there, four for dQ
 // and four for dK and dV, was measured level with this one.)
-template <bool BF, int D, int NKP>
+// FULL: the sequence length is a multiple of the 64 positions of a tile, so every lane's
+// position exists: no wave is switched off, no store is predicated, and the staged rows go to
+// LDS at the end of a tile's pass through the loop instead of at the top of the next.  The
+// compiler then knows how many stores lie between the loads of those rows and their use, and
+// the wait for the rows does not wait for the tile's stores as well (see fwd_mfma of the 2D
+// kernels).  Used at head_dim 128, where one workgroup per CU has nothing to cover that wait
+// with (B8 N8 T8192 k13: 229.6 -> 221 us; at head_dim 64 it measured 91.9 -> 92.2).
+template <bool BF, int D, int NKP, bool FULL = false>
 __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fused_mfma(
     BwdArgs a, int tiles_t, int ntiles) {
     using G = Geo1<D, NKP>;
@@ -501,7 +508,8 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
     zero_row1<D>(lds_k, NR, dlim);
     zero_row1<D>(lds_v, NR, dlim);
     if (threadIdx.x == 0) lds_stat[NR] = make_float2(0.f, 0.f);
-    const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, n = l & 15, g = l >> 4;
+    const int wave = FULL ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : threadIdx.x >> 6;
+    const int l = threadIdx.x & 63, n = l & 15, g = l >> 4;
     const float sc2 = s.scale * kLog2e;
     const int ntok = 15 + ks;
 
@@ -524,7 +532,7 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
     };
     Tile1 cur = tile1_of(sc.t, tiles_t, s.N);
     prefetch(cur);
-    for (;;) {
+    auto commit = [&]() __attribute__((always_inline)) {
         qst.commit(lds_q, dlim);
         gst.commit(lds_g, dlim);
         kst.commit(lds_k, dlim);
@@ -536,6 +544,10 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
             if (r < NR && threadIdx.x % CPR == 0) lds_stat[r].y = d;
         }
         if (threadIdx.x < NR) lds_stat[threadIdx.x].x = lse_st * kLog2e;
+    };
+    if constexpr (FULL) commit();
+    for (;;) {
+        if constexpr (!FULL) commit();
         __syncthreads();
         const int tn = sc.t + sc.step;
         const bool more = tn < sc.t_end;
@@ -543,10 +555,12 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
         if (more) {
             nxt = tile1_of(tn, tiles_t, s.N);
             prefetch(nxt);
+        } else {
+            if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the last tile (nothing is loaded, and the explicit wait says so to the compiler)
         }
         const int ra = row0_of(cur);
         const int w0 = cur.t0 + wave * 16;
-        if (w0 < T) {
+        if (FULL || w0 < T) {
             const bool live = w0 + n < T;
             const int pt = min(w0 + n, T - 1);  // this lane's position, as query and as key
             const int64_t goff = a.grad_at(cur.bb, cur.nn, 0, pt);
@@ -599,7 +613,7 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
                         dq[mt] = mfma16<BF>(cat(lds_read_tr(kp[0] + mt * 4), lds_read_tr(kp[1] + mt * 4)),
                                             dsb[kk], dq[mt]);
                 }
-                store_token<BF, D, D == 64 && !kNarrow>(static_cast<short *>(a.dq) + goff, g, dq, s.scale, live, dlim);
+                store_token<BF, D, D == 64 && !kNarrow, FULL>(static_cast<short *>(a.dq) + goff, g, dq, s.scale, live, dlim);
             }
             {
                 // ---- dK, dV: the queries that attend to any of the wave's 16 keys, 32 at a time
@@ -656,12 +670,16 @@ __global__ __launch_bounds__(256, D == 32 ? 3 : D == 64 ? 2 : 1) void bwd1d_fuse
                         dk[mt] = mfma16<BF>(cat(lds_read_tr(qt[0] + mt * 4), lds_read_tr(qt[1] + mt * 4)), dsb, dk[mt]);
                     }
                 }
-                store_token<BF, D, D == 64 && !kNarrow>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live, dlim);
-                store_token<BF, D, D == 64 && !kNarrow>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live, dlim);
+                store_token<BF, D, D == 64 && !kNarrow, FULL>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live, dlim);
+                store_token<BF, D, D == 64 && !kNarrow, FULL>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live, dlim);
             }
         }
-        if (!more) break;
+        if (!more) {
+            if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+            break;
+        }
         __syncthreads();
+        if constexpr (FULL) commit();
         cur = nxt;
         sc.t = tn;
     }
@@ -686,9 +704,13 @@ int bwd1d_fused_launch(const BwdArgs &a, hipStream_t st) {
     const int64_t nt = (int64_t)a.s.B * a.s.N * tiles_t;
     {
         ProfScope prof(ENATTEN_KERNEL_BWD_FUSED, "bwd1d_fused_mfma", st);
-        hipLaunchKernelGGL((bwd1d_fused_mfma<BF, D, NKP>),
-                           dim3(persistent_grid<bwd1d_fused_mfma<BF, D, NKP>>(nt)), dim3(256), 0, st, a,
-                           tiles_t, (int)nt);
+        const int grid = persistent_grid<bwd1d_fused_mfma<BF, D, NKP>>(nt);
+        constexpr bool kFull = !kNarrow && D == 128;
+        if (kFull && a.s.W % 64 == 0)
+            hipLaunchKernelGGL((bwd1d_fused_mfma<BF, D, NKP, kFull>), dim3(grid), dim3(256), 0, st, a, tiles_t,
+                               (int)nt);
+        else
+            hipLaunchKernelGGL((bwd1d_fused_mfma<BF, D, NKP>), dim3(grid), dim3(256), 0, st, a, tiles_t, (int)nt);
     }
     return check_launch("enatten1d_bwd");
 }
