@@ -504,7 +504,9 @@ struct HaloRegs {
 // stay in bounds and branch-free (the values only ever meet zero probabilities).
 // Addresses are a uniform base plus a 32-bit per-lane byte offset formed with
 // 24-bit multiplies: strides are below 2^22 elements (checked on the host).
-template <int D, int KS, int NW = 4, int SP = 1>
+// (I0, I1: only this thread's chunks I0 .. I1-1, for a kernel that loads the last chunks of a
+// halo behind its arithmetic because it has no registers for them beside it)
+template <int D, int KS, int NW = 4, int SP = 1, int I0 = 0, int I1 = Geo<D, KS, NW, SP>::NL>
 __device__ __forceinline__ void halo_fetch(HaloRegs<D, KS, NW, SP> &reg, const HaloPlan<D, KS, NW, SP> &pl,
                                   const short *img, int64_t sh, int64_t sw, int hr0, int hc0,
                                   int rlim, int clim) {
@@ -514,7 +516,7 @@ __device__ __forceinline__ void halo_fetch(HaloRegs<D, KS, NW, SP> &reg, const H
     const int rmax = rlim - 1 - hr0, cmax = clim - 1 - hc0;
     if (!pl.on) return;
 #pragma unroll
-    for (int i = 0; i < G::NL; i++) {
+    for (int i = I0; i < I1; i++) {
         const unsigned r = (unsigned)min(pl.rc[i] >> 8, rmax);
         const unsigned c = (unsigned)min(pl.rc[i] & 255, cmax);
         const unsigned off = __umul24(r, sh2) + __umul24(c, sw2) + (unsigned)pl.ch8 * 2u;

@@ -111,16 +111,21 @@ __device__ __forceinline__ void fetch32(Regs32 &reg, const float *img, int64_t s
 // matrix instructions (a wave that issues a whole halo at once is blocked for
 // microseconds while the CU's memory queue takes the loads, and issues no matrix
 // instruction meanwhile).
-template <int D, int KS, int PARTS>
+// TAIL: the last TAIL chunks of a thread are left out of the slices (part == PARTS loads them):
+// a kernel that has no registers for the whole halo beside its arithmetic loads them when the
+// arithmetic is over, instead of having the compiler spill freshly loaded chunks to scratch
+// memory, each behind a wait for its load.
+template <int D, int KS, int PARTS, int TAIL = 0>
 __device__ __forceinline__ void fetch32_part(Regs32 &reg, const float *img, int64_t sh, int64_t sw,
                                              int hr0, int hc0, int rlim, int clim, int part) {
     using G = Geo32<D, KS>;
+    static_assert(TAIL < G::NL, "the tail is a part of the halo");
     const char *base = reinterpret_cast<const char *>(img + hr0 * sh + hc0 * sw);
     const unsigned sh4 = (unsigned)sh * 4u, sw4 = (unsigned)sw * 4u;
     const int rmax = rlim - 1 - hr0, cmax = clim - 1 - hc0;
 #pragma unroll
     for (int i = 0; i < G::NL; i++) {
-        if (i * PARTS / G::NL != part) continue;
+        if ((i >= G::NL - TAIL ? PARTS : i * PARTS / (G::NL - TAIL)) != part) continue;
         int pix = (int)threadIdx.x / G::CPR + i * (256 / G::CPR);
         pix = pix < G::HR * G::HC ? pix : G::HR * G::HC - 1;
         const unsigned r = (unsigned)min(pix / G::HC, rmax), c = (unsigned)min(pix % G::HC, cmax);
@@ -388,6 +393,14 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_f32(FwdArgs a, int tiles_r, i
 // go to the workspace, k*k values per query in window order, for the dK/dV pass.
 // Persistent like the forward: K is loaded between the instructions of dP, the next
 // tile's V between those of dQ.
+// Chunks of a halo that the dQ pass loads behind its arithmetic (fetch32_part's TAIL), where it
+// would spill otherwise.  B4 N4 128x128 d128 k5: 84 -> 12 bytes of scratch per lane and
+// 261 -> 231 us; B4 N8 96x96 d32 k7: 76 -> 0 bytes, 194 -> 164 us; d64 k7: 288 -> 96 bytes,
+// 319 -> 273 us (the whole halo behind the arithmetic: its float64 logits of 13 token tiles
+// leave no registers for any of it).
+template <int D, int KS>
+constexpr int kDqTail = D == 128 && KS == 5 ? 5 : D == 32 && KS == 7 ? 5 : D == 64 && KS == 7 ? 12 : 0;
+
 template <int D, int KS>
 __global__ __launch_bounds__(256, 2) void bwd_dq_mfma_f32(BwdArgs a, float *ws_p, float *ws_ds,
                                                           int tiles_r, int tiles_c, int ntiles) {
@@ -419,7 +432,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_mfma_f32(BwdArgs a, float *ws_p
         float qf[G::DQ];
         float lse_f = 0.f;
         auto load_k = [&](int part) __attribute__((always_inline)) {
-            fetch32_part<D, KS, G::MT>(st, kimg, a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W, part);
+            fetch32_part<D, KS, G::MT, kDqTail<D, KS>>(st, kimg, a.k.sh, a.k.sw, lq.hr0, lq.hc0, s.H, s.W, part);
             if (part == G::MT - 1) {
                 load_quarter<D>(image32(a.q, cur) + lq.qr * a.q.sh + lq.qc * a.q.sw, g, qf);
                 lse_f = a.lse[lq.tok];
@@ -451,13 +464,14 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_mfma_f32(BwdArgs a, float *ws_p
 #pragma unroll
             for (int part = 0; part < G::MT; part++) load_k(part);
         }
+        if constexpr (kDqTail<D, KS> > 0) load_k(G::MT);
         const double lse = (double)lse_f;
         __syncthreads();  // every wave is done with V
         commit32<D, KS>(lds, st);
         __syncthreads();
         auto load_next = [&](int part) __attribute__((always_inline)) {
             if (more) {
-                fetch32_part<D, KS, STEPS>(st, vimg, a.v.sh, a.v.sw, lqn.hr0, lqn.hc0, s.H, s.W, part);
+                fetch32_part<D, KS, STEPS, kDqTail<D, KS>>(st, vimg, a.v.sh, a.v.sw, lqn.hr0, lqn.hc0, s.H, s.W, part);
                 if (part == STEPS - 1)
                     load_quarter<D>(image32(a.d_o, nxt) + lqn.qr * a.d_o.sh + lqn.qc * a.d_o.sw, g, go);
             }
@@ -510,6 +524,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_mfma_f32(BwdArgs a, float *ws_p
 #pragma unroll
             for (int part = 0; part < STEPS; part++) load_next(part);
         }
+        if constexpr (kDqTail<D, KS> > 0) load_next(STEPS);
         if (!more) break;
         __syncthreads();  // every wave is done with K
         cur = nxt;

@@ -558,6 +558,14 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void b
 //   phase 2  K rows in LDS: P from the saved log-sum-exp, delta, dS, dQ^T = K^T dS^T;
 //            the next tile's V rows are in flight meanwhile.
 // Four barriers per tile instead of two; 8x8 tiles, no column walk.
+// Chunks of a halo that bwd_dq2_mfma loads behind the arithmetic of a phase (see fetch_tail in
+// the kernel).  With 16x8 tiles at head_dim 128, kernel_size 13 a thread stages 18 chunks (72
+// registers) and the kernel spilled 70 registers, freshly loaded chunks among them, each spill
+// behind a wait for its load: B4 N4 128x128 167 us; with 8 chunks behind the arithmetic 125 us,
+// with 12 115.5, with 15 113.4 (5 registers spilled).  kernel_size 11: 16 chunks, 36 registers
+// spilled; with 8 chunks behind the arithmetic 110.6 us, with 13 107.5.
+template <int D, int KS, int NW>
+constexpr int kDq2Tail = D == 128 && NW == 8 ? (KS == 13 ? 15 : KS == 11 ? 13 : 0) : 0;
 // FULL: as in fwd_mfma.
 template <bool BF, int D, int KS, int NW = 4, bool FULL = false>
 __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS> : 1)) void bwd_dq2_mfma(BwdArgs a, TileSet ts, int ntiles) {
@@ -578,8 +586,15 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
     // phase ahead of phase 2: one spare set of row registers instead of two.
     s16x8 qreg[G::DS], gnext[G::DS];
     float lse_cur = 0.f;
+    // The last TAIL chunks of a halo are loaded when the arithmetic of the phase is over
+    // (fetch_tail): where the registers do not hold a whole halo beside it.
+    constexpr int TAIL = kDq2Tail<D, KS, NW>, HEAD = G::NL - TAIL;
     auto fetch_rows = [&](const View &vw, const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
-        halo_fetch<D, KS>(st, plan, image<short>(vw, tl), vw.sh, vw.sw, lq.hr0, lq.hc0, s.H, s.W);
+        halo_fetch<D, KS, NW, 1, 0, HEAD>(st, plan, image<short>(vw, tl), vw.sh, vw.sw, lq.hr0, lq.hc0, s.H, s.W);
+    };
+    auto fetch_tail = [&](const View &vw, const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
+        if constexpr (TAIL > 0)
+            halo_fetch<D, KS, NW, 1, HEAD, G::NL>(st, plan, image<short>(vw, tl), vw.sh, vw.sw, lq.hr0, lq.hc0, s.H, s.W);
     };
     auto fetch_do = [&](const Tile &tl, const LaneQ &lq) __attribute__((always_inline)) {
         load_row_chunks(gnext, image<short>(a.d_o, tl) + lq.qr * a.d_o.sh + lq.qc * a.d_o.sw, g, dlim);
@@ -592,6 +607,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
     Tile cur = tile_of(sc.t, ts.tiles_r, ts.tiles_c, s.N, G::TH);
     LaneQ lq = lane_query<KS>(cur, s, wave, n);
     fetch_rows(a.v, cur, lq);
+    fetch_tail(a.v, cur, lq);
     fetch_do(cur, lq);
     s16x8 greg[G::DS];
     // (V rows and the dO row at the end of a tile's pass through the loop, after its stores:
@@ -621,6 +637,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
                 dp[mt] = cp;
             }
         }
+        fetch_tail(a.k, cur, lq);
         __syncthreads();                      // every wave has read V
         halo_commit<D, KS>(lds_x, plan, st);  // K
         __syncthreads();
@@ -682,6 +699,7 @@ __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS>
             store_token<BF, D, kLineStores<D, KS, (NW == 4 ? kOneHaloWgs<D, KS> : 1)>, FULL>(static_cast<short *>(a.dq) + a.grad_at(cur.bb, cur.nn, lq.qr, lq.qc), g, dq, s.scale, lq.live, dlim);
             if (FULL || (lq.live && g == 0)) a.delta[lq.tok] = delta;
         }
+        if (more) fetch_tail(a.v, nxt, lqn);
         if (!more) {
             if constexpr (FULL) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), see fwd_mfma
             break;
@@ -1256,8 +1274,10 @@ constexpr bool kDq2Built = (D == 64 || D == 128) && Geo<D, KS>::WAVES == 1 && !k
 // workgroup of four waves per CU (head_dim 128, kernel_size 11 and 13) and the taller halo still
 // fits (128 and 153 KB): two waves per SIMD instead of one, and a quarter less halo per pixel.
 // B4 N4 128x128, us, 8x8 -> 16x8: forward k13 137.8 -> 104.5 (B8 N8: 526 -> 385), k11 143.4 -> 130.4;
-// dQ pass k13 179.7 -> 167.7 (B8 N8: 736 -> 642), k11 185.2 -> 190.4 (it spills 36 registers
-// there), so the dQ pass takes the tall tiles at kernel_size 13 only.
+// dQ pass k13 179.7 -> 167.7 (B8 N8: 736 -> 642), k11 185.2 -> 190.4 while it spilled 70 and 36
+// registers there; with the last chunks of a halo loaded behind the arithmetic (kDq2Tail) it
+// does not, and the tall tiles take k13 to 113 us and k11 to 107.5 (174 with 8x8 tiles; B8 N8:
+// 700 -> 426).
 template <int D, int KS>
 constexpr bool kFwd2TallBuilt = D == 128 && kOneHaloWgs<D, KS> == 1 && kOneHaloFits<D, KS> &&
                                 (size_t)Geo<D, KS, 8>::ROWS * Geo<D, KS, 8>::PITCH * 2 + 1024 <= 160 * 1024;
@@ -1265,7 +1285,7 @@ constexpr bool kFwd2TallBuilt = D == 128 && kOneHaloWgs<D, KS> == 1 && kOneHaloF
 // pass takes the 16x8 tiles too: one workgroup of eight waves instead of two of four, a quarter less halo
 // per pixel.  B2 N8 128x128 k13 81.5 -> 76.2 us, B4 N8 256x256 626 -> 606, B4 N4 128x128 k11 77.1 -> 76.3.
 template <int D, int KS>
-constexpr bool kDq2TallBuilt = (kFwd2TallBuilt<D, KS> && KS >= 13) || (D == 64 && KS >= 11);
+constexpr bool kDq2TallBuilt = kFwd2TallBuilt<D, KS> || (D == 64 && KS >= 11);
 template <int D, int KS>
 constexpr bool kFwd2Built = D == 128 && Geo<D, KS>::WAVES == 1 && kOneHaloFits<D, KS>;
 // Built at all: two halos fit, or the one-halo kernels serve the forward and the dQ pass and

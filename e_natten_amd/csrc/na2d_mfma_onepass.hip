@@ -91,8 +91,11 @@ __global__ __launch_bounds__(256, 2) void bwd_onepass_mfma(BwdArgs a, TileSet ts
         return static_cast<const short *>(vw.ptr) + tl.bb * vw.sb + tl.nn * vw.sn;
     };
     // The next tile's rows travel in two parts: q and k (and the log-sum-exp) while this
-    // tile's dQ is formed, v, dO and O while its dK and dV are formed, so that the registers
-    // of the second part are free during the first half of a tile.
+    // tile's dQ is formed, v, dO and O when its arithmetic is over.  Loaded earlier (while dK
+    // and dV are formed) they did not fit beside the accumulators at kernel_size 7 and at
+    // head_dim 64: the compiler spilled 24 and 38 registers, freshly loaded rows among them,
+    // each spill behind a wait for its load (B8 N2 112x112 d32 k7: 56.1 -> 53.3 us, B8 N8 28x28:
+    // 27.2 -> 25.2, B8 N4 56x56 d64 k3: 31.2 -> 30.0; nothing is spilled now).
     auto prefetch_qk = [&](const OTile &tl) __attribute__((always_inline)) {
         const int br = block_r(tl), bc = block_c(tl);
         halo_fetch<D, KS>(qst, plan, img(a.q, tl), a.q.sh, a.q.sw, br, bc, s.H, s.W);
@@ -200,9 +203,6 @@ __global__ __launch_bounds__(256, 2) void bwd_onepass_mfma(BwdArgs a, TileSet ts
             }
             store_token<BF, D>(static_cast<short *>(a.dq) + goff, g, dq, s.scale, live);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        if (more) prefetch_vgo(nxt);
-        __builtin_amdgcn_sched_barrier(0);
         {
             // ---- dK, dV: this lane's key is column n of every product
             s16x8 kreg[G::DS], vreg[G::DS];
@@ -332,6 +332,7 @@ __global__ __launch_bounds__(256, 2) void bwd_onepass_mfma(BwdArgs a, TileSet ts
             store_token<BF, D>(static_cast<short *>(a.dk) + goff, g, dk, s.scale, live);
             store_token<BF, D>(static_cast<short *>(a.dv) + goff, g, dv, 1.f, live);
         }
+        if (more) prefetch_vgo(nxt);
 
         if (!more) break;
         __syncthreads();  // every wave is done with this tile's LDS
