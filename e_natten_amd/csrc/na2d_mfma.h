@@ -707,13 +707,16 @@ int persistent_grid(int64_t ntiles, int threads = 256) {
 // an XCD on columns that are never neighbours at the same time; then the segments
 // are whole columns, or equal parts of a column, dealt out in turn, chosen for the
 // shortest walk of the busiest workgroup (a segment start costs about half a tile:
-// the whole halo is staged, not 8 rows of it).
-inline Runs plan_runs(int64_t ntiles, int grid, int colh) {
+// the whole halo is staged, not 8 rows of it).  `walk`, if given, receives that walk in
+// half tiles.
+inline Runs plan_runs(int64_t ntiles, int grid, int colh, double *walk = nullptr) {
     const int64_t slots = grid / 8, per = (ntiles + 7) / 8;
     const int64_t run = (per + slots - 1) / slots;
     Runs rp{(int)per, (int)run};
+    double best = 2.0 * run + 1.0;
+    if (walk) *walk = best;
     if (run <= colh) return rp;
-    double best = 1.3 * (2.0 * run + 1.0);  // measured: without the shared L2 lines, 1.3x the time
+    best *= 1.3;  // measured: without the shared L2 lines, 1.3x the time
     for (int m = 1; m <= 8; m++) {
         if (colh % m) continue;
         const int64_t seg = colh / m;
@@ -726,6 +729,7 @@ inline Runs plan_runs(int64_t ntiles, int grid, int colh) {
             rp.seg = (int)seg;
         }
     }
+    if (walk) *walk = best;
     return rp;
 }
 

@@ -1293,6 +1293,13 @@ constexpr bool kFwd2Built = D == 128 && Geo<D, KS>::WAVES == 1 && kOneHaloFits<D
 template <int D, int KS>
 constexpr bool kBuilt = fits<D, KS>() || (kFwd2Built<D, KS> && kDq2Built<D, KS>);
 
+// A frame tile's time in inner tiles in the dK/dV pass at head_dim 128, as the choice of the
+// split takes it (bwd_launch).  Measured over six image sizes from 64x64 to 256x256 with the
+// weights 0.8 to 4.0: 1.3 and 1.6 are within 1% of each other at k = 3, 5 and 7; at k = 9, where
+// the frame is two tiles wide, 2.0 is the best or within 3% of it everywhere (B4 N4 128x128: 227 us
+// with 1.15, 245 with 1.6, 176 with 2.0; B2 N2 256x256: 223, 167, 155).
+template <int KS>
+constexpr double kFrameCost128 = KS >= 9 ? 2.0 : KS == 5 ? 1.45 : 1.3;
 template <int D, int KS>
 constexpr int kDkdvSplit = D == 64 && Geo<D, KS>::WAVES == 1 ? 2 : 1;
 
@@ -1389,6 +1396,9 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         // inner tiles (no key or query within reach of the border) and frame
         TileSet ts;
         ts.tiles_r = tiles_r; ts.tiles_c = tiles_c;
+        // (tile row tr, keys 8 tr .. 8 tr + 7, is inner when no query with a clamped window
+        // attends to its keys: the queries of rows 0 .. k/2 - 1 reach the keys of rows 0 .. k - 1,
+        // so 8 tr >= k, and 8 tr + 7 <= H - 1 - k at the other end)
         ts.ir0 = (KS + 7) / 8; ts.ic0 = (KS + 7) / 8;
         ts.ni_r = (a.s.H - KS) / 8 - ts.ir0; ts.ni_c = (a.s.W - KS) / 8 - ts.ic0;
         if (ts.ni_r <= 0 || ts.ni_c <= 0 || kDkdvFrameOnly<D, KS>) {
@@ -1489,17 +1499,39 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             }
         }
         {
-            // Share the resident workgroups in proportion to the work.  Measured cost
-            // of a frame tile in inner tiles: about 2 when the inner tiles are bound
-            // by arithmetic (d <= 64), about 1.15 when they are bound by HBM (d = 128).
+            // Share the resident workgroups between the two bodies so that they end together.
+            // `cost` is a frame tile's time in inner tiles (measured): about 2 at head_dim <= 64
+            // (1.68 with the frame body's larger blocks), kFrameCost128 at head_dim 128.
             constexpr int SP = kDkdvSplit<D, KS>, NT = Geo<D, KS, 4, SP>::NT;
-            // (1.68 with the frame body's larger blocks: every weight from 1.6 to 1.75 gives the
-            // same split at 128x128)
-            const double cost = D >= 128 ? 1.15 : kFrameKS<D, KS, SP> != KS ? 1.68 : 2.0;
+            const double cost = D >= 128 ? kFrameCost128<KS> : kFrameKS<D, KS, SP> != KS ? 1.68 : 2.0;
             const int grid = persistent_grid<bwd_dkdv_mfma<BF, D, KS, false, SP>>(nb, NT);
             int inner_blocks = 0;
             if (n_frame == 0) {
                 inner_blocks = grid;
+            } else if (n_inner > 0 && kRollBuilt<D>) {
+                // With the column walk the busiest inner workgroup's walk is a staircase in the
+                // number of inner workgroups (plan_runs), and a share in proportion to the work
+                // lands anywhere on a step.  So every split is tried: the fewest inner
+                // workgroups among those whose longer side is shortest.
+                double best = 1e30;
+                const int64_t per_f = (n_frame + 7) / 8, per_i = (n_inner + 7) / 8;
+                for (int ib = 8; ib <= grid - 8 && ib <= per_i * 8; ib += 8) {
+                    double walk;
+                    if (roll_pays<D>(n_inner, ib)) {
+                        plan_runs(n_inner, ib, ts.ni_r, &walk);
+                    } else {
+                        const int64_t slots_i = ib / 8;
+                        walk = 2.0 * (double)((per_i + slots_i - 1) / slots_i);
+                    }
+                    const int64_t slots_f = (grid - ib) / 8;
+                    const double frame = 2.0 * cost * (double)((per_f + slots_f - 1) / slots_f);
+                    const double t = walk > frame ? walk : frame;
+                    if (t < best) {
+                        best = t;
+                        inner_blocks = ib;
+                    }
+                }
+                if (inner_blocks == 0) inner_blocks = 8;
             } else if (n_inner > 0) {
                 const double f = (double)n_inner / ((double)n_inner + cost * (double)n_frame);
                 inner_blocks = (int)(f * grid / 8.0 + 0.5) * 8;
