@@ -957,7 +957,7 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
 template <bool BF, int D, int KS, int SP, int KSG, bool RED_OVER>
 __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, int ntiles,
                                            int block, int nblocks, short *lds_q, short *lds_g,
-                                           float2 *lds_stat, f32x4 *lds_red) {
+                                           float4 *lds_stat, f32x4 *lds_red) {
     using G = Geo<D, KSG, 4, SP>;
     const Shape &s = a.s;
     const int dlim = kNarrow ? s.D : D;  // head dim of the tensors: D, or less in the build for narrow dims
@@ -1029,8 +1029,13 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 #pragma unroll
         for (int i = 0; i < G::NST; i++) {
             const int id = threadIdx.x + i * G::NT;
-            if (id < G::ZROW) lds_stat[id] = sst[i];
-            else if (id == G::ZROW) lds_stat[id] = make_float2(0.f, 0.f);
+            // per staged query: lse * log2e, delta, and where its window starts (row in the low,
+            // column in the high half of a word), so that the mask of a logit is two
+            // differences; the padding row's window is nowhere
+            const int r = min(cur.br + id / G::HC, cur.qb - 1), c = min(cur.bc + id % G::HC, cur.cb - 1);
+            const int ws = win_start(r, s.H, KS) | (win_start(c, s.W, KS) << 16);
+            if (id < G::ZROW) lds_stat[id] = make_float4(sst[i].x, sst[i].y, __int_as_float(ws), 0.f);
+            else if (id == G::ZROW) lds_stat[id] = make_float4(0.f, 0.f, __int_as_float(0x7fff7fff), 0.f);
         }
         if (cur.first) {
 #pragma unroll
@@ -1086,13 +1091,10 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         const int qi = q0 + m2 * 16 + g * 4 + i;
-                        const int dvd = (qi * magic) >> 16;
-                        const int er = ra + dvd, ec = cc + qi - dvd * wcols;
-                        const float2 st = lds_stat[row_of(qi)];
-                        const bool ok =
-                            (qi < nq) &
-                            ((unsigned)(kr - win_start(er, s.H, KS)) < (unsigned)KS) &
-                            ((unsigned)(kc - win_start(ec, s.W, KS)) < (unsigned)KS);
+                        const float4 st = lds_stat[row_of(qi)];
+                        const int ws = __float_as_int(st.z);
+                        const bool ok = ((unsigned)(kr - (ws & 0xffff)) < (unsigned)KS) &
+                                        ((unsigned)(kc - (ws >> 16)) < (unsigned)KS);
                         const float p =
                             __builtin_amdgcn_exp2f(ok ? cs[i] * sc2 - st.x : -INFINITY);
                         pb[m2 * 4 + i] = cvt16<BF>(p);
@@ -1193,7 +1195,7 @@ __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) v
     constexpr size_t I_ROWS = FRAME_ONLY ? 0 : (size_t)G::ROWS * G::PITCH * sizeof(short);
     constexpr size_t F_ROWS = (size_t)FG::ROWS * FG::PITCH * sizeof(short);
     constexpr size_t I_STAT = FRAME_ONLY ? 0 : (G::ROWS * sizeof(float2) + 15) / 16 * 16;
-    constexpr size_t F_STAT = (FG::ROWS * sizeof(float2) + 15) / 16 * 16;
+    constexpr size_t F_STAT = FG::ROWS * sizeof(float4);
     constexpr size_t I_ALL = 2 * I_ROWS + I_STAT + RED;
     constexpr size_t F_ALL = 2 * F_ROWS + F_STAT + (RED_OVER ? 0 : RED);
     static_assert(RED <= F_ROWS || !RED_OVER, "the partial sums lie over the staged Q rows");
@@ -1217,7 +1219,7 @@ __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) v
     {
         short *lds_q = reinterpret_cast<short *>(lds_raw);
         short *lds_g = reinterpret_cast<short *>(lds_raw + F_ROWS);
-        float2 *lds_stat = reinterpret_cast<float2 *>(lds_raw + 2 * F_ROWS);
+        float4 *lds_stat = reinterpret_cast<float4 *>(lds_raw + 2 * F_ROWS);
         f32x4 *lds_red = reinterpret_cast<f32x4 *>(RED_OVER ? lds_raw : lds_raw + 2 * F_ROWS + F_STAT);
         dkdv_frame<BF, D, KS, SP, kFrameKS<D, KS, SP>, RED_OVER>(
             a, ts, n_frame, blockIdx.x - inner_blocks, gridDim.x - inner_blocks, lds_q, lds_g,
@@ -1602,7 +1604,8 @@ int bwd_dispatch(const BwdArgs &a, int dtype, int path, hipStream_t st) {
     auto al = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
     const bool grads_ok = a.gsb % 8 == 0 && a.gsn % 8 == 0 && a.gsh % 8 == 0 && a.gsw % 8 == 0;
     if (!layout_ok(a.q) || !layout_ok(a.k) || !layout_ok(a.v) || !layout_ok(a.o) ||
-        !layout_ok(a.d_o) || !al(a.dq) || !al(a.dk) || !al(a.dv) || !grads_ok)
+        !layout_ok(a.d_o) || !al(a.dq) || !al(a.dk) || !al(a.dv) || !grads_ok ||
+        a.s.H >= 32768 || a.s.W >= 32768)  // (the dK/dV pass keeps window starts in 16 bits)
         return launch_bwd_simt(a, dtype, st);
     if (dtype == ENATTEN_BF16) {
         ENATTEN_BY_D(bwd_launch, true, a, path, st)
