@@ -1502,10 +1502,12 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         }
         {
             // Share the resident workgroups between the two bodies so that they end together.
-            // `cost` is a frame tile's time in inner tiles (measured): about 2 at head_dim <= 64
-            // (1.68 with the frame body's larger blocks), kFrameCost128 at head_dim 128.
+            // `cost` is a frame tile's time in inner tiles (measured): 2 at head_dim 64 (1.68 with
+            // the frame body's larger blocks), 2.5 at head_dim 32 (against 2: B8 N2 112x112 k7
+            // 28.7 -> 27.1 us, B8 N4 56x56 20.8 -> 18.6, B4 N4 128x128 k5 27.1 -> 25.4, k3 23.1 ->
+            // 21.5; 2-4% slower at 96x96 and 256x256 k7), kFrameCost128 at head_dim 128.
             constexpr int SP = kDkdvSplit<D, KS>, NT = Geo<D, KS, 4, SP>::NT;
-            const double cost = D >= 128 ? kFrameCost128<KS> : kFrameKS<D, KS, SP> != KS ? 1.68 : 2.0;
+            const double cost = D >= 128 ? kFrameCost128<KS> : kFrameKS<D, KS, SP> != KS ? 1.68 : D == 32 ? 2.5 : 2.0;
             const int grid = persistent_grid<bwd_dkdv_mfma<BF, D, KS, false, SP>>(nb, NT);
             int inner_blocks = 0;
             if (n_frame == 0) {
