@@ -12,6 +12,7 @@ ABI_VERSION = 5  # ENATTEN_ABI_VERSION of include/enatten.h
 F32, BF16, F16, F64 = 0, 1, 2, 3
 STATIC_BWD_MAX_QUERIES = 1 << 20
 PATH_NONE, PATH_SIMT, PATH_MFMA, PATH_MFMA_FUSED, PATH_MFMA_SPLIT = 0, 1, 2, 3, 4
+PATH_MFMA_SPLIT_QUEUE = 5
 
 _lock = threading.Lock()
 _lib = None

@@ -145,7 +145,7 @@ int enatten2d_kernel_path(int D, int kernel_size, int dtype) {
 
 int enatten_set_path(int path) {
     if (path != 0 && path != ENATTEN_PATH_SIMT && path != ENATTEN_PATH_MFMA_FUSED &&
-        path != ENATTEN_PATH_MFMA_SPLIT)
+        path != ENATTEN_PATH_MFMA_SPLIT && path != ENATTEN_PATH_MFMA_SPLIT_QUEUE)
         return g_path.load();
     return g_path.exchange(path);
 }

@@ -777,7 +777,7 @@ int bwd1d_dispatch(const BwdArgs &a, int dtype, int path, hipStream_t st) {
     if (!layout1d_ok(a.q) || !layout1d_ok(a.k) || !layout1d_ok(a.v) || !layout1d_ok(a.d_o) ||
         !al(a.dq) || !al(a.dk) || !al(a.dv) || a.gsb % 8 != 0 || a.gsn % 8 != 0 || a.gsw % 8 != 0)
         return launch_bwd_simt(a, dtype, st);
-    if (path != ENATTEN_PATH_MFMA_SPLIT && fused1d_supported(a)) {
+    if (!split_forced(path) && fused1d_supported(a)) {
         ENATTEN_1D(bwd1d_fused_launch, a, dtype, st)
     }
     ENATTEN_1D(bwd1d_launch, a, dtype, st)

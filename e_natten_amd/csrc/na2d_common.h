@@ -129,7 +129,11 @@ int launch_bwd_mfma_f32(const BwdArgs &a, hipStream_t st);
 bool mfma_supported(int D, int ks, int dtype);
 int launch_fwd_mfma(const FwdArgs &a, int dtype, hipStream_t st);
 // `path`: 0 chooses between the two-pass and the fused backward, ENATTEN_PATH_MFMA_FUSED /
-// ENATTEN_PATH_MFMA_SPLIT force one of them
+// ENATTEN_PATH_MFMA_SPLIT force one of them (ENATTEN_PATH_MFMA_SPLIT_QUEUE: the two passes,
+// the dK/dV pass dealing its frame tiles from a counter)
+inline bool split_forced(int path) {
+    return path == ENATTEN_PATH_MFMA_SPLIT || path == ENATTEN_PATH_MFMA_SPLIT_QUEUE;
+}
 int launch_bwd_mfma(const BwdArgs &a, int dtype, int path, hipStream_t st);
 // the same kernels built for head dims that are multiples of 8 below the next of 32, 64, 128
 int launch_fwd_mfma_narrow(const FwdArgs &a, int dtype, hipStream_t st);

@@ -379,6 +379,8 @@ constexpr int kDqWaves = D == 32 && (KS == 7 || KS == 9) && NW == 4 ? 3 : Geo<D,
 // the end of a tile's pass through the loop).
 template <bool BF, int D, int KS, bool FRAME, bool ROLL, int NW = 4, bool FULL = false>
 __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (kDqWaves<D, KS, NW>)) void bwd_dq_mfma(BwdArgs a, TileSet ts, int ntiles, Runs rp) {
+    // (the dK/dV pass that follows on the stream counts its frame tiles here, from zero)
+    if (blockIdx.x == 0 && threadIdx.x == 0 && a.zinv) *reinterpret_cast<int *>(a.zinv) = 0;
     using G = Geo<D, KS, NW>;
     __shared__ __attribute__((aligned(16))) short lds_k[G::ROWS * G::PITCH];
     __shared__ __attribute__((aligned(16))) short lds_v[G::ROWS * G::PITCH];
@@ -569,6 +571,8 @@ constexpr int kDq2Tail = D == 128 && NW == 8 ? (KS == 13 ? 15 : KS == 11 ? 13 : 
 // FULL: as in fwd_mfma.
 template <bool BF, int D, int KS, int NW = 4, bool FULL = false>
 __global__ __launch_bounds__((Geo<D, KS, NW>::NT), (NW == 4 ? kOneHaloWgs<D, KS> : 1)) void bwd_dq2_mfma(BwdArgs a, TileSet ts, int ntiles) {
+    // (the dK/dV pass that follows on the stream counts its frame tiles here, from zero)
+    if (blockIdx.x == 0 && threadIdx.x == 0 && a.zinv) *reinterpret_cast<int *>(a.zinv) = 0;
     using G = Geo<D, KS, NW>;
     __shared__ __attribute__((aligned(16))) short lds_x[G::ROWS * G::PITCH];
     const Shape &s = a.s;
@@ -957,11 +961,27 @@ __device__ __forceinline__ void dkdv_inner(const BwdArgs &a, const TileSet &ts, 
 template <bool BF, int D, int KS, int SP, int KSG, bool RED_OVER>
 __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, int ntiles,
                                            int block, int nblocks, short *lds_q, short *lds_g,
-                                           float4 *lds_stat, f32x4 *lds_red) {
+                                           float4 *lds_stat, f32x4 *lds_red, int *tile_ctr, int *lds_tile) {
     using G = Geo<D, KSG, 4, SP>;
     const Shape &s = a.s;
     const int dlim = kNarrow ? s.D : D;  // head dim of the tensors: D, or less in the build for narrow dims
+    // Tiles: a strided share of the XCD's run (make_sched), or, with a counter in device memory
+    // that is zero when the kernel starts (`tile_ctr`), whatever tile is next when the workgroup
+    // is free.  A workgroup then knows its tile and the one after it, and asks for the tile after
+    // those while it works on a tile's first block, so the answer never holds it up.
+    const bool dyn = tile_ctr != nullptr;
     Sched sc = make_sched(ntiles, block, nblocks);
+    int t_next = sc.t + sc.step;
+    if (dyn) {
+        if (threadIdx.x == 0) {
+            lds_tile[0] = atomicAdd(tile_ctr, 1);
+            lds_tile[1] = atomicAdd(tile_ctr, 1);
+        }
+        __syncthreads();
+        sc.t = lds_tile[0];
+        t_next = lds_tile[1];
+        sc.t_end = ntiles;
+    }
     if (sc.t >= sc.t_end) return;
     zero_row<D, KSG, 4, SP>(lds_q, dlim);
     zero_row<D, KSG, 4, SP>(lds_g, dlim);
@@ -1024,6 +1044,8 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
     stage(cur);
     load_keys(cur.tl);
     for (;;) {
+        int fetched = 0;
+        if (dyn && cur.first && threadIdx.x == 0) fetched = atomicAdd(tile_ctr, 1);
         halo_commit<D, KSG>(lds_q, plan, qst);
         halo_commit<D, KSG>(lds_g, plan, gst);
 #pragma unroll
@@ -1048,8 +1070,8 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
 
         KeyBlock nxt = cur;
         bool more = next_block<G::HR, G::HC>(nxt);
-        if (!more && cur.t + sc.step < sc.t_end) {
-            nxt = first_of(cur.t + sc.step);
+        if (!more && t_next < sc.t_end) {
+            nxt = first_of(t_next);
             more = true;
         }
         if constexpr (SP > 1) {
@@ -1118,6 +1140,9 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
             }
         }
 
+        // (read below, behind the barrier that ends this block; the first block of the next tile
+        // writes it again behind the barrier that opens its arithmetic)
+        if (dyn && cur.first && threadIdx.x == 0) lds_tile[0] = fetched;
         const bool live = (wr0 + (n >> 2) < s.H) && (wc0 + (n & 3) < s.W);
         auto store = [&]() __attribute__((always_inline)) {
             const int64_t goff = a.grad_at(cur.tl.bb, cur.tl.nn, kr, kc);
@@ -1154,6 +1179,7 @@ __device__ __forceinline__ void dkdv_frame(const BwdArgs &a, const TileSet &ts, 
             if (!more) break;
             if (RED_OVER && cur.last) __syncthreads();  // the sums are read: the next block may land
         }
+        if (nxt.first) t_next = dyn ? lds_tile[0] : nxt.t + sc.step;  // the tile after the next one
         cur = nxt;
     }
 }
@@ -1182,7 +1208,7 @@ constexpr int kDkdvWaves =
     SP == 1 && D <= 64 && 3 * (Geo<D, KS>::LDS_BYTES + 2048) <= 160 * 1024 ? 3 : Geo<D, KS, 4, SP>::WAVES;
 template <bool BF, int D, int KS, bool ROLL, int SP = 1>
 __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) void bwd_dkdv_mfma(
-    BwdArgs a, TileSet ts, int n_inner, int n_frame, int inner_blocks, Runs rp) {
+    BwdArgs a, TileSet ts, int n_inner, int n_frame, int inner_blocks, Runs rp, int dyn) {
     using G = Geo<D, KS, 4, SP>;
     using FG = Geo<D, kFrameKS<D, KS, SP>, 4, SP>;  // blocks of the frame body
     // One LDS buffer, laid out by each body for itself: staged Q rows, staged dO rows,
@@ -1201,6 +1227,11 @@ __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) v
     static_assert(RED <= F_ROWS || !RED_OVER, "the partial sums lie over the staged Q rows");
     __shared__ __attribute__((aligned(16))) char lds_raw[I_ALL > F_ALL ? I_ALL : F_ALL];
     static_assert(sizeof(lds_raw) <= 160 * 1024, "LDS");
+    // dyn: the frame tiles are dealt out as workgroups become free, the inner workgroups joining
+    // when their walk is over; the counter lies where the general kernels keep 1 / Z per query,
+    // and the dQ pass, which runs before this one on the stream, has cleared it.
+    __shared__ int lds_tile[2];
+    int *tile_ctr = dyn ? reinterpret_cast<int *>(a.zinv) : nullptr;
     if constexpr (!FRAME_ONLY) {
         if ((int)blockIdx.x < inner_blocks) {
             short *lds_q = reinterpret_cast<short *>(lds_raw);
@@ -1213,7 +1244,8 @@ __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) v
             else  // the same number of barriers as the first part
                 dkdv_inner<BF, D, KS, ROLL, SP, SP - 1>(a, ts, n_inner, rp, blockIdx.x, inner_blocks,
                                                         lds_q, lds_g, lds_stat, lds_red);
-            return;
+            if (!dyn) return;
+            __syncthreads();
         }
     }
     {
@@ -1222,8 +1254,8 @@ __global__ __launch_bounds__((Geo<D, KS, 4, SP>::NT), (kDkdvWaves<D, KS, SP>)) v
         float4 *lds_stat = reinterpret_cast<float4 *>(lds_raw + 2 * F_ROWS);
         f32x4 *lds_red = reinterpret_cast<f32x4 *>(RED_OVER ? lds_raw : lds_raw + 2 * F_ROWS + F_STAT);
         dkdv_frame<BF, D, KS, SP, kFrameKS<D, KS, SP>, RED_OVER>(
-            a, ts, n_frame, blockIdx.x - inner_blocks, gridDim.x - inner_blocks, lds_q, lds_g,
-            lds_stat, lds_red);
+            a, ts, n_frame, dyn ? blockIdx.x : blockIdx.x - inner_blocks,
+            dyn ? gridDim.x : gridDim.x - inner_blocks, lds_q, lds_g, lds_stat, lds_red, tile_ctr, lds_tile);
     }
 }
 
@@ -1412,7 +1444,7 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         // The fused backward wherever it is built (fused_bwd_supported): 5-25% faster than the
         // two passes at every size measured, from B64 N16 8x8 (45.7 against 47.3 us) and B4 N4
         // 32x32 (14.8 against 24.1) to B16 N8 128x128 (938 against 1174).
-        if (path != ENATTEN_PATH_MFMA_SPLIT && fused_bwd_supported(a)) {
+        if (!split_forced(path) && fused_bwd_supported(a)) {
             const int rc = launch_bwd_fused(a, BF, ts, nb, st);
             return rc ? rc : check_launch("enatten2d_bwd");
         }
@@ -1429,7 +1461,7 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
         // 56x56 52.7 vs 49.0.  So it is the default only where at most one tile in eight is an
         // inner tile (level with the two passes there, one launch less);
         // ENATTEN_PATH_MFMA_FUSED forces it wherever it is built.
-        if (path != ENATTEN_PATH_MFMA_SPLIT && onepass_bwd_supported(a) &&
+        if (!split_forced(path) && onepass_bwd_supported(a) &&
             (path == ENATTEN_PATH_MFMA_FUSED || 8 * n_inner <= nb)) {
             const int rc = launch_bwd_onepass(a, BF, ts, nb, st);
             return rc ? rc : check_launch("enatten2d_bwd");
@@ -1509,7 +1541,7 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
             constexpr int SP = kDkdvSplit<D, KS>, NT = Geo<D, KS, 4, SP>::NT;
             const double cost = D >= 128 ? kFrameCost128<KS> : kFrameKS<D, KS, SP> != KS ? 1.68 : D == 32 ? 2.5 : 2.0;
             const int grid = persistent_grid<bwd_dkdv_mfma<BF, D, KS, false, SP>>(nb, NT);
-            int inner_blocks = 0;
+            int inner_blocks = 0, dyn = 0;
             if (n_frame == 0) {
                 inner_blocks = grid;
             } else if (n_inner > 0 && kRollBuilt<D>) {
@@ -1536,6 +1568,29 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
                     }
                 }
                 if (inner_blocks == 0) inner_blocks = 8;
+                // The other way to share: every workgroup walks inner tiles (the shortest walk
+                // there is) and then takes frame tiles from a counter as it becomes free.  The
+                // frame tiles then run at the end, next to no inner tile and in no XCD's order,
+                // which costs where the static split is already even; it is taken where the
+                // staircase leaves the static split 7% or more behind (B4 N4 128x128 k7: 154.6 ->
+                // 135.4 us; measured 4-9% slower at k9 and at 256x256 and 96x96 k7, where it is
+                // not taken).
+                if (a.zinv != nullptr) {
+                    int all = grid;
+                    if (all > per_i * 8) all = (int)(per_i * 8);
+                    double walk;
+                    if (roll_pays<D>(n_inner, all)) {
+                        plan_runs(n_inner, all, ts.ni_r, &walk);
+                    } else {
+                        const int64_t slots_i = all / 8;
+                        walk = 2.0 * (double)((per_i + slots_i - 1) / slots_i);
+                    }
+                    const double t_dyn = walk + 2.0 * cost * ((double)n_frame / grid + 1.0);
+                    if (t_dyn < 0.93 * best) {
+                        dyn = 1;
+                        inner_blocks = all;
+                    }
+                }
             } else if (n_inner > 0) {
                 const double f = (double)n_inner / ((double)n_inner + cost * (double)n_frame);
                 inner_blocks = (int)(f * grid / 8.0 + 0.5) * 8;
@@ -1543,14 +1598,19 @@ int bwd_launch(const BwdArgs &a, int path, hipStream_t st) {
                 if (inner_blocks > grid - 8) inner_blocks = grid - 8;
                 if (inner_blocks > (n_inner + 7) / 8 * 8) inner_blocks = (int)((n_inner + 7) / 8 * 8);
             }
+            if (path == ENATTEN_PATH_MFMA_SPLIT_QUEUE && a.zinv != nullptr && n_frame > 0 && !dyn) {
+                dyn = 1;
+                const int64_t all = (n_inner + 7) / 8 * 8;
+                inner_blocks = all < grid ? (int)all : grid;
+            }
             ProfScope prof(ENATTEN_KERNEL_BWD_DKDV, "bwd_dkdv_mfma", st);
             if (inner_blocks > 0 && roll_pays<D>(n_inner, inner_blocks))
                 hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, kRollBuilt<D>, SP>), dim3(grid), dim3(NT),
                                    0, st, a, ts, (int)n_inner, (int)n_frame, inner_blocks,
-                                   plan_runs(n_inner, inner_blocks, ts.ni_r));
+                                   plan_runs(n_inner, inner_blocks, ts.ni_r), dyn);
             else
                 hipLaunchKernelGGL((bwd_dkdv_mfma<BF, D, KS, false, SP>), dim3(grid), dim3(NT), 0, st,
-                                   a, ts, (int)n_inner, (int)n_frame, inner_blocks, Runs{0, 0});
+                                   a, ts, (int)n_inner, (int)n_frame, inner_blocks, Runs{0, 0}, dyn);
         }
         return check_launch("enatten2d_bwd");
     } else {

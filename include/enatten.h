@@ -43,7 +43,8 @@ enum {
 
 /* which kernel family a call is routed to (enatten2d_kernel_path) */
 enum { ENATTEN_PATH_NONE = 0, ENATTEN_PATH_SIMT = 1, ENATTEN_PATH_MFMA = 2,
-       ENATTEN_PATH_MFMA_FUSED = 3, ENATTEN_PATH_MFMA_SPLIT = 4 /* enatten_set_path only */ };
+       ENATTEN_PATH_MFMA_FUSED = 3, ENATTEN_PATH_MFMA_SPLIT = 4 /* enatten_set_path only */,
+       ENATTEN_PATH_MFMA_SPLIT_QUEUE = 5 /* enatten_set_path only */ };
 
 int enatten_abi_version(void);
 
@@ -64,7 +65,10 @@ int enatten2d_kernel_path(int D, int kernel_size, int dtype);
  * kernel_size 5, image sides that are multiples of 8; the 1D operator has one for
  * kernel_size <= 17, and for head_dim <= 64 beyond).  Automatic dispatch and
  * ENATTEN_PATH_MFMA_FUSED take the fused form wherever it is built (it was measured
- * faster at every size), ENATTEN_PATH_MFMA_SPLIT never.
+ * faster at every size), ENATTEN_PATH_MFMA_SPLIT never.  ENATTEN_PATH_MFMA_SPLIT_QUEUE is
+ * ENATTEN_PATH_MFMA_SPLIT with the dK/dV pass dealing its border tiles from a counter as
+ * workgroups become free wherever it has any (automatic dispatch does that where its cost
+ * model says it pays).
  * Process-wide; meant for tests and tuning.  Returns the previous setting.
  */
 int enatten_set_path(int path);

@@ -87,6 +87,29 @@ def test_fused_backward_path(shape, dtype, _lib):
 
 
 @pytest.mark.parametrize("shape,ks,dtype", [
+    ((2, 3, 56, 72, 128), 7, BF),     # one workgroup per CU, inner columns walked, then frame tiles from the counter
+    ((1, 2, 64, 48, 128), 9, F16),    # frame two tiles wide
+    ((1, 1, 40, 56, 128), 13, BF),    # no inner body: every tile from the counter, 12x12 blocks
+    ((2, 4, 64, 72, 64), 13, BF),     # two waves per block of keys, 22x22 frame blocks, sums through LDS
+    ((4, 4, 56, 56, 32), 7, BF),      # three workgroups per CU
+    ((1, 2, 37, 50, 64), 5, F16),     # ragged sides
+    ((1, 1, 16, 16, 128), 5, BF),     # fewer tiles than workgroups ask for
+])
+def test_dkdv_frame_tiles_from_the_counter(shape, ks, dtype, _lib):
+    # the two-pass backward with the dK/dV pass dealing its frame tiles from the counter in
+    # the workspace (automatic dispatch does so only at sizes the oracle does not reach),
+    # twice in a row: the second call finds the first call's count in whatever memory it
+    # gets and relies on its own dQ pass to clear it
+    from e_natten_amd._lib import PATH_MFMA_SPLIT_QUEUE
+    prev = _lib.enatten_set_path(PATH_MFMA_SPLIT_QUEUE)
+    try:
+        _case(shape, dtype, ks, what="frame tiles from the counter %s" % (shape,))
+        _case(shape, dtype, ks, seed=1, what="frame tiles from the counter, second call %s" % (shape,))
+    finally:
+        _lib.enatten_set_path(prev)
+
+
+@pytest.mark.parametrize("shape,ks,dtype", [
     ((8, 16, 16, 64, 128), 5, BF),    # several short columns per workgroup: whole columns in turn
     ((32, 8, 32, 32, 128), 5, BF),    # the same with taller columns
     ((4, 10, 128, 128, 128), 5, F16), # quarter columns in turn
@@ -577,18 +600,20 @@ def test_tensors_beyond_2_31_elements(dtype, _lib):
     torch.cuda.empty_cache()
 
 
-def test_full_size_invariants():
-    # properties that need no oracle, at the benchmark's full size:
+@pytest.mark.parametrize("ks", [5, 7])
+def test_full_size_invariants(ks):
+    # properties that need no oracle, at the benchmark's full size (kernel_size 7: the size at
+    # which automatic dispatch has the dK/dV pass deal its frame tiles from the counter):
     # rows of P sum to 1  => sum_keys dV == sum_queries dO
     # sum_j dS_j = 0      => dK summed over keys is zero up to rounding
     # constant V          => O equals that constant
     q, k, v, g = make_inputs((4, 4, 128, 128, 128), BF, 1)
-    o, dq, dk, dv = run_gpu(q, k, v, g, 5)
+    o, dq, dk, dv = run_gpu(q, k, v, g, ks)
     tot = g.float().sum((2, 3))
     assert ((dv.float().sum((2, 3)) - tot).abs().max() / tot.abs().max()) < 2e-2
     assert dk.float().sum((2, 3)).abs().max() / dk.float().abs().sum((2, 3)).max() < 2e-2
     vc = torch.full_like(v, 1.5)
-    oc = run_gpu(q, k, vc, g, 5)[0]
+    oc = run_gpu(q, k, vc, g, ks)[0]
     assert (oc.float() - 1.5).abs().max() < 2e-2
 
 
